@@ -55,8 +55,10 @@ def read_config_json(model_dir: str) -> dict[str, Any]:
 
 def architecture_of(raw: dict[str, Any]) -> str:
     archs = raw.get("architectures")
+    if not archs and isinstance(raw.get("architecture"), str):
+        return raw["architecture"]              # the one-name spelling some designs use
     if not archs or not isinstance(archs, (list, tuple)) or not isinstance(archs[0], str):
-        raise ConfigError("config.json must name the model class in 'architectures': [\"...\"]")
+        raise ConfigError("config.json must name the model class in 'architectures': [\"...\"] (or 'architecture': \"...\")")
     return archs[0]
 
 
@@ -238,3 +240,136 @@ class Qwen3Config:
         """Sizes as a flat dict (for benchmark records)."""
         return {f.name: getattr(self, f.name) for f in fields(self)
                 if f.name not in ("layer_types",)}
+
+
+# ------------------------------------------------------------------------------------ Sigosun
+
+@dataclass(frozen=True)
+class SigosunLayer:
+    """One entry of a Sigosun config's `layers`: which mixer, the mixer's sizes and constants as the file
+    gives them (validated, with the optional keys resolved), and the feed-forward width (None: no feed-forward)."""
+
+    kind: str                  # "attention", "mamba2" or "lightning"
+    mixer: dict
+    ff: int | None
+
+
+@register_config("Sigosun")
+@dataclass(frozen=True)
+class SigosunConfig:
+    """The ``config.json`` keys of the Sigosun design: a list of layers, each with its own mixer (softmax
+    attention under a block mask, a selective state-space recurrence, or linear attention with fixed decays),
+    sizes and constants, and an optional dense feed-forward; one norm eps; vocabulary and width. Every size
+    and constant comes from the file: nothing of a particular model is assumed."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple
+    eos_token_id: int | None = None
+    max_position_embeddings: int | None = None
+
+    MIXER_KEYS = {
+        "attention": (("heads", int), ("kv_heads", int), ("dim", int), ("vdim", int), ("scale", float)),
+        "mamba2": (("heads", int), ("vdim", int), ("state", int), ("groups", int), ("conv", int), ("norm_groups", int)),
+        "lightning": (("heads", int), ("dim", int), ("vdim", int)),
+    }
+
+    @classmethod
+    def from_dict(cls, raw: dict[str, Any]) -> "SigosunConfig":
+        norm = raw.get("norm")
+        if not isinstance(norm, dict):
+            raise ConfigError("config.json lacks the object 'norm'")
+        listed = raw.get("layers")
+        if not isinstance(listed, list) or not listed:
+            raise ConfigError("config.json lacks the list 'layers'")
+        layers = []
+        for i, entry in enumerate(listed):
+            where = f"layers[{i}]"
+            kind = entry.get("type") if isinstance(entry, dict) else None
+            if kind not in cls.MIXER_KEYS:
+                raise ConfigError(f"{where}: 'type' must be one of {sorted(cls.MIXER_KEYS)}, got {kind!r}")
+            m = entry.get("mixer")
+            if not isinstance(m, dict):
+                raise ConfigError(f"{where} lacks the object 'mixer'")
+            mixer = {key: _need(m, key, typ, where + ".mixer") for key, typ in cls.MIXER_KEYS[kind]}
+            if kind == "attention":
+                rot, mask = m.get("rot"), m.get("mask")
+                mixer["rot_dims"] = _need(rot, "dims", int, where + ".mixer.rot") if rot else 0
+                mixer["rot_base"] = _need(rot, "base", float, where + ".mixer.rot") if rot else 1.0
+                mixer["mask_size"] = _need(mask, "size", int, where + ".mixer.mask") if mask else None
+                mixer["kv_from"] = m.get("kv_from")
+            elif kind == "lightning":
+                decay = m.get("decay")
+                if not isinstance(decay, list) or len(decay) != mixer["heads"]:
+                    raise ConfigError(f"{where}.mixer: 'decay' must list one number per head")
+                mixer["decay"] = tuple(float(d) for d in decay)
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{where}.mlp: only kind 'dense' is known, got {mlp.get('kind')!r}")
+                ff = _need(mlp, "ff", int, where + ".mlp")
+            layers.append(SigosunLayer(kind, mixer, ff))
+        cfg = cls(vocab_size=_need(raw, "vocab", int), hidden_size=_need(raw, "width", int),
+                  norm_eps=_need(norm, "eps", float, "config.json norm"), layers=tuple(layers),
+                  eos_token_id=raw.get("eos_token_id"), max_position_embeddings=raw.get("max_position_embeddings"))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.norm_eps > 0:
+            raise ConfigError("vocab and width must be positive and norm.eps above zero")
+        for i, layer in enumerate(self.layers):
+            m, where = layer.mixer, f"layers[{i}]"
+            if any(isinstance(v, int) and not isinstance(v, bool) and v < 1 for k, v in m.items()
+                   if k not in ("rot_dims", "kv_from", "mask_size")):
+                raise ConfigError(f"{where}: sizes must be positive")
+            if layer.kind == "attention":
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"{where}: {m['heads']} heads are not a multiple of {m['kv_heads']} kv_heads")
+                if m["rot_dims"] % 2 or not 0 <= m["rot_dims"] <= m["dim"]:
+                    raise ConfigError(f"{where}: rot.dims must be even and at most dim")
+                if m["mask_size"] is not None and m["mask_size"] < 1:
+                    raise ConfigError(f"{where}: mask.size must be positive")
+                src = m["kv_from"]
+                if src is not None:
+                    if not (isinstance(src, int) and 0 <= src < i and self.layers[src].kind == "attention"
+                            and self.layers[src].mixer["kv_from"] is None):
+                        raise ConfigError(f"{where}: kv_from must name an earlier attention layer that has keys of its own")
+                    o = self.layers[src].mixer
+                    if any(o[k] != m[k] for k in ("kv_heads", "dim", "vdim")):
+                        raise ConfigError(f"{where}: kv_from names a layer with other key/value sizes")
+            elif layer.kind == "mamba2":
+                if m["heads"] % m["groups"] or (m["heads"] * m["vdim"]) % m["norm_groups"]:
+                    raise ConfigError(f"{where}: heads must be a multiple of groups, and heads * vdim of norm_groups")
+            if layer.ff is not None and layer.ff < 1:
+                raise ConfigError(f"{where}.mlp: ff must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        """A ``config.json`` that reads back to an equal config."""
+        out = []
+        for layer in self.layers:
+            m = dict(layer.mixer)
+            if layer.kind == "attention":
+                dims, base, size, src = m.pop("rot_dims"), m.pop("rot_base"), m.pop("mask_size"), m.pop("kv_from")
+                if dims:
+                    m["rot"] = {"dims": dims, "base": base}
+                if size is not None:
+                    m["mask"] = {"size": size}
+                if src is not None:
+                    m["kv_from"] = src
+            elif layer.kind == "lightning":
+                m["decay"] = list(m["decay"])
+            out.append({"type": layer.kind, "mixer": m, "mlp": None if layer.ff is None else {"kind": "dense", "ff": layer.ff}})
+        d = {"architecture": self.architecture_name, "vocab": self.vocab_size, "width": self.hidden_size,
+             "norm": {"eps": self.norm_eps}, "layers": out}
+        if self.eos_token_id is not None:
+            d["eos_token_id"] = self.eos_token_id
+        if self.max_position_embeddings is not None:
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d
+
+    def flat(self) -> dict[str, Any]:
+        return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
+                "layer_kinds": [layer.kind for layer in self.layers]}

@@ -58,6 +58,7 @@ struct AttnArgs {
   int page, page_shift;         // page = 1 << page_shift
   float scale;
   int window;                   // 0: all keys
+  int chunk;                    // > 0: a block mask (only the keys of the query's own block of `chunk` positions); window is then huge
   int tok_tile;                 // prefill: query tokens per workgroup
   int part_size;                // decode: keys per partition (multiple of 32)
   int num_parts;                // decode: partitions launched
@@ -85,6 +86,12 @@ struct AttnArgs {
   bf16_t* v_cache_w;
 };
 
+// The first key a query at `pos` sees when there is a lower edge at all (a.window > 0): its block's first position
+// under a block mask, else the window's. Both grow with pos, which is all the kernels assume of it.
+__device__ __forceinline__ int lower_edge(const AttnArgs& a, int pos) {
+  return a.chunk > 0 ? pos - pos % a.chunk : max(0, pos - a.window + 1);
+}
+
 // Key range of the tile that holds new token `tl` (index within its sequence's new tokens) and the
 // number of segments it is cut into; shared by the prefill kernel and the merge kernel.
 struct TileRange {
@@ -95,7 +102,7 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tok0, int
   const int start = L - q_len;
   r.tok0 = tok0;
   r.tile_tokens = min(a.tok_tile, q_len - tok0);
-  r.tile_lo = a.window > 0 ? max(0, start + tok0 - a.window + 1) : 0;
+  r.tile_lo = a.window > 0 ? lower_edge(a, start + tok0) : 0;
   r.tile_base = r.tile_lo & ~31;
   r.pos_last = start + tok0 + r.tile_tokens - 1;
   // never more than the scratch has room for: the last segment then runs to the tile's end
@@ -479,13 +486,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       head[ct] = kvh * a.G + hh;
       const int pos = start + tok0 + tl;
       col_hi[ct] = valid[ct] ? pos : -1;
-      col_lo[ct] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+      col_lo[ct] = a.window > 0 ? lower_edge(a, pos) : 0;
       load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
     }
     // keys this wave needs: from the window start of its first column to its last column's position
     const int c_last = min(ncols, c0 + 16 * CT) - 1;
     const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
-    const int w_lo = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+    const int w_lo = a.window > 0 ? lower_edge(a, pos_first) : 0;
     float m[CT], l[CT];
     f32x4 acc[CT][DT];
 #pragma unroll
@@ -497,7 +504,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // a block all of whose keys every column of this wave sees (below the first column's position,
     // above the last column's window start) needs no masks
     const int full_hi = pos_first - 31;                                   // t0 <= full_hi: all 32 keys visible
-    const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;  // t0 >= full_lo: none behind a window
+    const int full_lo = a.window > 0 ? lower_edge(a, pos_last) : 0;  // t0 >= full_lo: none behind a window
     // One set of key registers and one of value registers, refilled as soon as the products that
     // read them are issued: the next keys arrive behind the softmax and the value product, the next
     // values behind the score product and the softmax. Page ids are looked up a block earlier
@@ -778,13 +785,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       head[ct] = kvh * a.G + hh;
       const int pos = start + tok0 + tl;
       col_hi[ct] = valid[ct] ? pos : -1;
-      col_lo[ct] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+      col_lo[ct] = a.window > 0 ? lower_edge(a, pos) : 0;
       load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
     }
     const int c_last = min(ncols, c0 + 16 * CT) - 1;
     const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
     const int full_hi = active ? pos_first - 31 : -(1 << 30);
-    const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;
+    const int full_lo = a.window > 0 ? lower_edge(a, pos_last) : 0;
     float m[CT], l[CT];
     f32x4 acc[CT][DT];
 #pragma unroll
@@ -1076,13 +1083,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
       head[ct] = kvh * a.G + hh;
       const int pos = start + tok0 + tl;
       col_hi[ct] = valid[ct] ? pos : -1;
-      col_lo[ct] = WINDOW ? max(0, pos - a.window + 1) : 0;
+      col_lo[ct] = WINDOW ? lower_edge(a, pos) : 0;
       load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
     }
     const int c_last = min(ncols, c0 + 16 * CT) - 1;
     const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
     const int full_hi = active ? pos_first - 31 : -(1 << 30);
-    const int full_lo = WINDOW ? max(0, pos_last - a.window + 1) : 0;
+    const int full_lo = WINDOW ? lower_edge(a, pos_last) : 0;
     float m[CT], l[CT];
     f32x4 acc[CT][DT];
 #pragma unroll
@@ -1286,7 +1293,7 @@ __global__ void __launch_bounds__(256) attn_prefill_merge_kernel(AttnArgs a, int
 // of contexts of very different lengths the longest sequences start first instead of last.
 // =====================================================================================
 __device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int& first, int& end) {
-  const int lo = a.window > 0 ? max(0, L - a.window) : 0;
+  const int lo = a.window > 0 ? lower_edge(a, L - 1) : 0;
   first = min((lo & ~31) / a.part_size, a.num_parts - 1);
   end = max(first + 1, min(a.num_parts, (L + a.part_size - 1) / a.part_size));
 }
@@ -1323,7 +1330,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     if (part < first || part >= end) return;
   }
   const int pos = L - 1;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = a.window > 0 ? lower_edge(a, pos) : 0;
   const int32_t* bt = a.block_tables + (int64_t)b * a.bt_stride;
   const int ncols = min(16, a.G - ctile * 16);
   const bool valid = n < ncols;
@@ -1586,7 +1593,7 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   ME_CHECK((reinterpret_cast<uintptr_t>(q) % 16 == 0) && (reinterpret_cast<uintptr_t>(out) % 8 == 0) &&
                (reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) && (reinterpret_cast<uintptr_t>(v_cache) % 16 == 0),
            "attention: q, out and cache pointers must be 16-byte aligned");
-  ME_CHECK(window >= 0 && bt_stride >= 1, "attention: bad window or block-table stride");
+  ME_CHECK(bt_stride >= 1, "attention: bad block-table stride");
   ME_CHECK(scale > 0.f, "attention: the score scale must be positive");
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
   a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
@@ -1594,7 +1601,9 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   a.cu_seqlens = nullptr; a.num_seqs = num_seqs; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv;
   a.page = page; a.page_shift = 0;
   while ((1 << a.page_shift) < page) ++a.page_shift;
-  a.scale = scale; a.window = window; a.tok_tile = 1; a.part_size = 0; a.num_parts = 1; a.spread_heads = 1;
+  a.scale = scale; a.tok_tile = 1;
+  // a negative window names a block mask of that many positions; the kernels then take their windowed paths
+  a.chunk = window < 0 ? -window : 0; a.window = window < 0 ? (1 << 30) : window; a.part_size = 0; a.num_parts = 1; a.spread_heads = 1;
   a.tmp_out = a.tmp_m = a.tmp_l = nullptr;
   a.seg_keys = 0; a.max_segs = 1; a.pf_scratch = nullptr; a.seq_of_token = nullptr; a.seq_base = 0;
   a.raw_k = a.raw_v = nullptr; a.q_w = a.k_w = nullptr; a.eps = 0.f; a.rope = nullptr;
@@ -1642,7 +1651,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
     const bool three = ct == 2 && waves == 3;
 #define DMA_LAUNCH(CTV, WV)                                                                                    \
   do {                                                                                                         \
-    if (window > 0) attn_prefill_dma_kernel<CTV, WV, true><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);  \
+    if (window != 0) attn_prefill_dma_kernel<CTV, WV, true><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);  \
     else attn_prefill_dma_kernel<CTV, WV, false><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);            \
   } while (0)
     if (three) DMA_LAUNCH(2, 3); else if (ct == 2) DMA_LAUNCH(2, 2); else DMA_LAUNCH(1, 2);

@@ -41,7 +41,8 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
   // keys [lo, hi): up to the query's own position, never past the request's context (a padding
   // row has context 0 and sees nothing)
   const int hi = min(pos + 1, context_lens[b]);
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  // window > 0: the last `window` keys; window < 0: a block mask, only the keys of the query's own block of -window positions
+  const int lo = window > 0 ? max(0, pos - window + 1) : (window < 0 ? pos - pos % (-window) : 0);
   float m = -INFINITY, l = 0.f;
   // thread d < D owns output channel d (two channels per thread when D > AS_THREADS)
   float acc0 = 0.f, acc1 = 0.f;
@@ -111,7 +112,7 @@ extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_
   if (num_tokens == 0) return 0;
   ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   ME_CHECK(D >= 1 && D <= 2 * AS_THREADS, "attention (float32 path): head_dim %d outside 1..%d", D, 2 * AS_THREADS);
-  ME_CHECK(page >= 1 && window >= 0, "attention: bad page size or window");
+  ME_CHECK(page >= 1, "attention: bad page size");
   dim3 grid(num_tokens, Hq), block(AS_THREADS);
   size_t lds = (size_t)(D + AS_THREADS) * sizeof(float);
   if (dtype == ME_F32)

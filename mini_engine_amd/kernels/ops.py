@@ -19,6 +19,8 @@ import torch
 from . import build
 
 ME_BF16, ME_F32 = 0, 1
+ACTIVATIONS = {"silu": 0, "relu2": 1}          # elementwise activations of `activation`
+GATED_NORMS = {"silu_before": 0, "sigmoid_behind": 1}
 _DT = {torch.bfloat16: ME_BF16, torch.float32: ME_F32}
 
 
@@ -68,6 +70,13 @@ _CORE_PROTOS = {
     "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
+    "me_add_rms_norm": [P, I, I, L, P, P, P, P, L, I, F, P],
+    "me_add_rms_norm_partials": [P, I, L, P, P, P, P, L, I, F, P],
+    "me_activation": [P, L, P, I, I, L, I, P],
+    "me_head_gate": [P, P, L, I, L, I, I, P],
+    "me_causal_conv": [P, L, I, P, P, P, L, P, P, P, P, L, I, I, I, P],
+    "me_linear_recurrence": [P, L, P, L, P, L, I, P, L, P, P, P, P, P, L, P, P, P, L, I, I, I, I, I, I, I, I, P, P],
+    "me_gated_rms_norm": [P, I, L, P, L, I, P, P, L, I, I, I, F, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
 }
@@ -304,8 +313,11 @@ class HipBackend:
     def paged_attention(self, q, k_cache, v_cache, page: int, block_tables, context_lens, seq_of_token,
                         positions, prefill_cu, num_decodes: int, max_decode_context: int, scale: float,
                         window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False,
-                        max_prefill_context: int = 0, even_contexts: bool = False, decode_as_prefill: bool = False):
-        """Causal attention of this step's tokens over the paged keys of their requests.
+                        max_prefill_context: int = 0, even_contexts: bool = False, decode_as_prefill: bool = False,
+                        chunk: int | None = None):
+        """Causal attention of this step's tokens over the paged keys of their requests. `chunk`: a block mask in
+        place of a window: the query at position i sees the keys j <= i of its own block, floor(j / chunk) =
+        floor(i / chunk) (the kernels take it as a negative window).
 
         q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
         each, `num_decodes` of them), then the others; `prefill_cu` int32 [B - num_decodes + 1]
@@ -329,7 +341,9 @@ class HipBackend:
         _check(_is_i32(context_lens) and _is_i32(seq_of_token, T) and _is_i32(positions, T), "attention: metadata must be int32")
         _check(0 <= num_decodes <= B and num_decodes <= T, "attention: bad decode count")
         out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
-        win = int(window or 0)
+        _check(not (window and chunk), "attention: a window and a block mask exclude each other")
+        win = -int(chunk) if chunk else int(window or 0)
+        span = abs(win)          # no query sees more keys than this (0: all of them)
         mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8 and page & (page - 1) == 0
                 and not force_simple)
         if not mfma:
@@ -355,8 +369,8 @@ class HipBackend:
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
             Tp = T - num_decodes
-            col_tiles = prefill_col_tiles(max_prefill_context, win, Tp, Hq, D)
-            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D, col_tiles)
+            col_tiles = prefill_col_tiles(max_prefill_context, span, Tp, Hq, D)
+            seg_keys, max_segs = prefill_segments(max_prefill_context, span, Tp, Hq, D, col_tiles)
             waves = prefill_waves(max_prefill_context, Tp, B - num_decodes, Hq, Hkv, col_tiles, max_segs)
             # the segments' partial results: in a buffer that is kept between steps (a step's decode rows have
             # finished with theirs before, on the same stream, but the two are kept apart all the same)
@@ -371,7 +385,7 @@ class HipBackend:
 
     def decode_step_attention(self, qkv, q_weight, k_weight, eps, table, k_cache, v_cache, page: int, block_tables,
                               context_lens, max_context: int, scale: float, window: int | None, Hq: int, Hkv: int,
-                              D: int, even_contexts: bool = False):
+                              D: int, even_contexts: bool = False, chunk: int | None = None):
         """A pure decode step's `qk_norm_rope_store` and `paged_attention` as one launch: rows [B, (Hq+2Hkv)*D]
         as the packed product left them (row r is request r's one new token, at position context_lens[r] - 1).
         The kernel norms and rotates q and the new key in float32, rounds them to bfloat16 as the separate
@@ -404,7 +418,8 @@ class HipBackend:
         attn_lib(D).call("me_attn_decode_fused", qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0),
                          _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
                          k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
-                         context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale), int(window or 0),
+                         context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale),
+                         -int(chunk) if chunk else int(window or 0),
                          part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, _stream())
         return out
 
@@ -556,6 +571,115 @@ class HipBackend:
         core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                     ME_BF16, None, 1, M, N, inter, 1, 0, 0, _stream())
         return y
+
+    # -- norms on a sublayer's output, activations, gates ----------------------------------
+    def add_rms_norm(self, y: torch.Tensor, weight: torch.Tensor, eps: float, stream: torch.Tensor, out_dtype: torch.dtype):
+        """stream + weight * y / sqrt(mean(y^2) + eps), all float32. y: [T, n] in the compute dtype, or float32
+        partial sums [P, T, n] that are added first. Returns (the new stream rounded to out_dtype, the new stream
+        float32 [T, n]); with out_dtype float32 both are one tensor."""
+        parts = y.shape[0] if y.dim() == 3 else 1
+        _check(y.is_contiguous() and (y.dim() == 2 or y.dtype == torch.float32), "add_rms_norm: y contiguous, partial sums float32")
+        T, n = y.shape[-2], y.shape[-1]
+        _check(weight.dtype == torch.float32 and weight.shape == (n,) and weight.is_contiguous(), "add_rms_norm: weight float32 [n]")
+        _check(stream.dtype == torch.float32 and stream.shape == (T, n) and stream.is_contiguous(), "add_rms_norm: stream float32 [T, n]")
+        new = torch.empty_like(stream)
+        if out_dtype == torch.float32:
+            _check(y.dtype == torch.float32, "add_rms_norm: a float32 stream copy needs float32 rows")
+            core().call("me_add_rms_norm", y.data_ptr(), ME_F32, parts, T * n, weight.data_ptr(), stream.data_ptr(), new.data_ptr(),
+                        None, T, n, float(eps), _stream())
+            return new, new
+        rounded = torch.empty((T, n), dtype=out_dtype, device=y.device)
+        if y.dtype == torch.float32:
+            core().call("me_add_rms_norm_partials", y.data_ptr(), parts, T * n, weight.data_ptr(), stream.data_ptr(), new.data_ptr(),
+                        rounded.data_ptr(), T, n, float(eps), _stream())
+        else:
+            core().call("me_add_rms_norm", y.data_ptr(), _code(y.dtype), 1, 0, weight.data_ptr(), stream.data_ptr(), new.data_ptr(),
+                        rounded.data_ptr(), T, n, float(eps), _stream())
+        return rounded, new
+
+    def activation(self, x: torch.Tensor, kind: str) -> torch.Tensor:
+        """silu(x) or relu(x)^2 of a row view [T, n] (unit inner stride), float32 inside; contiguous result."""
+        _check(x.dim() == 2 and x.stride(1) == 1 and kind in ACTIVATIONS, "activation: rows with unit inner stride, a known kind")
+        T, n = x.shape
+        out = torch.empty((T, n), dtype=x.dtype, device=x.device)
+        core().call("me_activation", x.data_ptr(), x.stride(0), out.data_ptr(), _code(x.dtype), ACTIVATIONS[kind], T, n, _stream())
+        return out
+
+    def head_gate(self, o: torch.Tensor, gate: torch.Tensor, H: int, D: int) -> None:
+        """o[t, h, :] *= sigmoid(gate[t, h]) in place; o contiguous [T, H * D], gate a view [T, H]."""
+        T = o.shape[0]
+        _check(o.is_contiguous() and o.shape == (T, H * D) and gate.shape == (T, H) and gate.stride(1) == 1
+               and gate.dtype == o.dtype, "head_gate: o [T, H * D] contiguous, gate [T, H] of its dtype")
+        core().call("me_head_gate", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(o.dtype), T, H, D, _stream())
+
+    # -- mixers with a state of fixed size -------------------------------------------------
+    def causal_conv(self, x, weight, bias, state, state_slots, cu_seqlens, seq_of_token) -> torch.Tensor:
+        """silu(bias + sum_j weight[:, j] * x[t - (taps - 1) + j]) per channel over every request's tokens of this step,
+        continued from its state: x a row view [T, C]; weight float32 [C, taps] (the last tap is the current
+        token's); state a float32 view [slots, C * (taps - 1)] (per channel the inputs before the request's next
+        token, oldest first), rows `state_slots`; it moves on by this step's tokens. Returns [T, C]."""
+        T, C = x.shape
+        taps = weight.shape[1]
+        B = state_slots.numel()
+        _check(x.stride(1) == 1 and weight.dtype == torch.float32 and weight.shape == (C, taps) and weight.is_contiguous()
+               and bias.dtype == torch.float32 and bias.shape == (C,) and bias.is_contiguous(), "causal_conv: bad operands")
+        _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] == C * (taps - 1),
+               "causal_conv: state must be float32 [slots, C * (taps - 1)]")
+        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and _is_i32(seq_of_token, T), "causal_conv: metadata must be int32")
+        out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+        core().call("me_causal_conv", x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), bias.data_ptr(),
+                    state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_of_token.data_ptr(),
+                    out.data_ptr(), T, B, C, taps, _stream())
+        return out
+
+    def linear_recurrence(self, q, k, v, state, state_slots, cu_seqlens, q_lens, H: int, G: int, N: int, P: int,
+                          decay=None, dt=None, dt_bias=None, rate=None, skip=None) -> torch.Tensor:
+        """Per request and head, over the request's tokens of this step in order, from its state row:
+            S_t = a_t S_(t-1) + b_t k_t v_t^T,   y_t = S_t^T q_t (+ skip_h v_t),      S [N, P] float32.
+        q, k: row views [T, G * N] (heads share them by groups of H / G), v: [T, H * P]; state: float32 view
+        [slots, H * N * P], rows `state_slots`, left at the state behind the last token. a, b: `decay` (float32 [H])
+        and 1; or exp(-rate_h dt), dt with dt = softplus(dt[t, h] + dt_bias_h) (`dt` a row view [T, H], the others
+        float32 [H]). `q_lens`: the requests' token counts on the host: long ones are cut into spans that run side
+        by side (`recurrence_spans`). Returns float32 [T, H * P], or partial sums [S, T, H * P] over slices of N
+        for a consumer that adds them."""
+        T, B = v.shape[0], state_slots.numel()
+        dtype = v.dtype
+        for t, width in ((q, G * N), (k, G * N), (v, H * P)):
+            _check(t.dim() == 2 and t.shape == (T, width) and t.stride(1) == 1 and t.dtype == dtype, "recurrence: bad q, k or v rows")
+        _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] == H * N * P,
+               "recurrence: state must be float32 [slots, H * N * P]")
+        _check((decay is None) != (dt is None), "recurrence: fixed decays or step sizes")
+        for w in (decay, dt_bias, rate, skip):
+            _check(w is None or (w.dtype == torch.float32 and w.shape == (H,) and w.is_contiguous()), "recurrence: per-head constants float32 [H]")
+        if dt is not None:
+            _check(dt.shape == (T, H) and dt.stride(1) == 1 and dt.dtype == dtype and dt_bias is not None and rate is not None,
+                   "recurrence: step sizes [T, H] with bias and rates")
+        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B, "recurrence: metadata")
+        per_wave = recurrence_rows_per_wave(N)
+        slices = -(-N // per_wave)
+        span, spans = recurrence_spans(q_lens, H * -(-P // 64) * slices)
+        scratch = _scratch(B * spans * (H * N * P + H), v.device, "recurrence") if spans > 1 else None
+        y = torch.empty((slices, T, H * P) if slices > 1 else (T, H * P), dtype=torch.float32, device=v.device)
+        core().call("me_linear_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                    _code(dtype), _ptr(dt), 0 if dt is None else dt.stride(0), _ptr(decay), _ptr(dt_bias), _ptr(rate), _ptr(skip),
+                    state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), y.data_ptr(), T * H * P,
+                    B, H, G, N, P, per_wave, span, spans, _ptr(scratch), _stream())
+        return y
+
+    def gated_rms_norm(self, y, gate, weight, eps: float, groups: int, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+        """`kind` "silu_before": u = y * silu(gate), out = u / rms(u) * weight with the root mean square taken over
+        each of `groups` equal parts of a row; "sigmoid_behind": out = y / rms(y) * weight * sigmoid(gate). y float32
+        [T, n] or slices [S, T, n] that are added first; gate a row view [T, n] of out_dtype. Returns [T, n]."""
+        parts = y.shape[0] if y.dim() == 3 else 1
+        T, n = y.shape[-2], y.shape[-1]
+        _check(y.dtype == torch.float32 and y.is_contiguous() and kind in GATED_NORMS, "gated_rms_norm: float32 rows, a known kind")
+        _check(gate.shape == (T, n) and gate.stride(1) == 1 and gate.dtype == out_dtype, "gated_rms_norm: gate [T, n] of the output dtype")
+        _check(weight.dtype == torch.float32 and weight.shape == (n,) and weight.is_contiguous() and n % groups == 0,
+               "gated_rms_norm: weight float32 [n], n a multiple of the groups")
+        out = torch.empty((T, n), dtype=out_dtype, device=y.device)
+        core().call("me_gated_rms_norm", y.data_ptr(), parts, T * n, gate.data_ptr(), gate.stride(0), _code(out_dtype),
+                    weight.data_ptr(), out.data_ptr(), T, n, groups, GATED_NORMS[kind], float(eps), _stream())
+        return out
 
     # -- sampling ------------------------------------------------------------------------
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
@@ -968,6 +1092,37 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     return part, parts
 
 
+def recurrence_rows_per_wave(N: int) -> int:
+    """State rows a wave of the recurrence kernel keeps in registers per lane (16, 32, 48 or 64): all of N up to 64,
+    beyond that the size that wastes the fewest rows over its slices (ties to the larger)."""
+    if N <= 64:
+        return -(-N // 16) * 16
+    return min((64, 48, 32), key=lambda r: (-(-N // r) * r - N, -r))
+
+
+RECURRENCE_MIN_SPAN = 64
+RECURRENCE_WAVES = 2048        # waves that keep the 256 compute units busy: 8 a unit
+
+
+def recurrence_spans(q_lens: list, waves_per_request: int) -> tuple:
+    """(tokens per span, most spans per request) for the recurrence kernel; (0, 1): every request in one pass.
+
+    A request's tokens are a chain, and one pass gives the GPU only requests x heads x slices waves. A long prompt is
+    therefore cut into spans that run side by side: each span first from zero, then a walk over the spans' end states
+    carries the state on, then each span again from the state before it, which costs the work twice and pays as soon
+    as the spans are many. Spans of RECURRENCE_MIN_SPAN tokens or more, as many as bring the launch to
+    RECURRENCE_WAVES waves, for steps whose longest request has two spans or more."""
+    longest = max(q_lens, default=0)
+    if longest < 2 * RECURRENCE_MIN_SPAN:
+        return 0, 1
+    total = sum(q_lens)
+    want = max(1, RECURRENCE_WAVES // max(1, waves_per_request))        # spans over all requests
+    span = max(RECURRENCE_MIN_SPAN, -(-total // want))
+    span = -(-span // 16) * 16
+    spans = -(-longest // span)
+    return (span, spans) if spans >= 2 else (0, 1)
+
+
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     """Whether `rows` rows against the packed gate/up weight w [2 I, K] are few enough, and w of a kind, for the
     gating to happen in the product's epilogue: a bfloat16 product that the unsplit skinny kernel takes, up to
@@ -1065,3 +1220,9 @@ def silu_mul_linear(*a, **k): return backend().silu_mul_linear(*a, **k)
 def norm_linear(*a, **k): return backend().norm_linear(*a, **k)
 def gated_linear(*a, **k): return backend().gated_linear(*a, **k)
 def sample(*a, **k): return backend().sample(*a, **k)
+def add_rms_norm(*a, **k): return backend().add_rms_norm(*a, **k)
+def activation(*a, **k): return backend().activation(*a, **k)
+def head_gate(*a, **k): return backend().head_gate(*a, **k)
+def causal_conv(*a, **k): return backend().causal_conv(*a, **k)
+def linear_recurrence(*a, **k): return backend().linear_recurrence(*a, **k)
+def gated_rms_norm(*a, **k): return backend().gated_rms_norm(*a, **k)

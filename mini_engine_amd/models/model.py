@@ -11,7 +11,7 @@ from dataclasses import dataclass
 import torch
 
 from ..kernels import ops
-from ..parts.base import CacheNeed, LayerCall, Part, StateNeed
+from ..parts.base import CacheNeed, LayerCall, Part, Settled, StateNeed
 from ..parts.block import norm_of
 
 
@@ -108,6 +108,9 @@ class DecoderModel(Part):
         """Final norm of (h + residual), then the rows that want logits, then the head: float32
         [len(rows), vocab] (reference models/qwen3.py:91,116-117; layers/embed_head.py:19-23).
         `out`: where the head puts them (`parts.Head.forward(x, out)`)."""
+        if isinstance(h, Settled):          # the last layer has added its output to the stream already: wanted rows first
+            x, _ = self.final_norm.forward(ops.gather_rows(residual, rows), None)
+            return self.head.forward(x, out=out)
         x, _ = norm_of(self.final_norm, h, residual)
         x = ops.gather_rows(x, rows)
         return self.head.forward(x, out=out)

@@ -2,6 +2,10 @@
 layers/attention.py:43-76)."""
 from __future__ import annotations
 
+import math
+
+import torch
+
 from ..kernels import ops
 from .base import CacheNeed, Mixer, ParamSpec, PositionEncoding, register_part
 from .linear import Linear
@@ -17,13 +21,25 @@ class Attention(Mixer):
     Consecutive query heads share a key/value head: kv head = q head // (Hq/Hkv).
     `own_kv=False` builds a mixer with queries only, for a layer call that reads the cache
     another call has written.
+
+    Further options, all off by default: `value_dim` (values of another size than queries and keys),
+    `chunk` (a block mask: the query at position i sees the keys j <= i with floor(j / chunk) = floor(i / chunk),
+    blocks counted from position 0 of the request), `head_gate` (each head's output is multiplied by the
+    sigmoid of one more output feature of the packed product, one per head), and a position encoding that
+    wants the heads laid out differently from how they are stored (`PositionEncoding.head_order`: partial or
+    interleaved rotations). The parameters are declared as they are stored (q, k, v and gate rows, heads of
+    `head_dim` and `value_dim`); where the kernels need another layout (one head size for keys and values, a
+    multiple of 16; the rotation's pairs half a head apart; rows in steps of 8), `finalize` builds it once: rows
+    reordered within each head, zero rows and columns where a head is padded, the norm weights scaled so that a
+    mean over the padded head equals the mean over the stored one.
     """
 
     takes_pending_norm = True      # x goes to the packed product and nowhere else
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, qk_norm_eps: float | None = None, position: PositionEncoding | None = None,
-                 window: int | None = None, own_kv: bool = True):
+                 window: int | None = None, own_kv: bool = True, value_dim: int | None = None,
+                 chunk: int | None = None, head_gate: bool = False):
         super().__init__()
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
@@ -35,18 +51,39 @@ class Attention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = window
         self.own_kv = own_kv
+        if window is not None and chunk is not None:
+            raise ValueError("a trailing window and a block mask exclude each other")
+        self.chunk = chunk
+        self.head_gate = bool(head_gate)
+        self.stored_dim = head_dim
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
+        order = position.head_order() if position is not None and hasattr(position, "head_order") else None
+        slots = getattr(position, "head_dim", head_dim) if position is not None else head_dim
+        if self.value_dim != head_dim or slots != head_dim:
+            # one head size for the kernels: the larger of the two, in whole steps of 16
+            head_dim = self.head_dim = max(slots, -(-max(head_dim, self.value_dim) // 16) * 16)
+            if position is not None and slots != head_dim:
+                raise ValueError(f"the position encoding must be built for the kernels' head size {head_dim}")
+        self._relayout = order is not None or head_dim != self.stored_dim or head_dim != self.value_dim
         self.q_size = num_heads * head_dim
         self.kv_size = num_kv_heads * head_dim
+        stored_q, stored_k, stored_v = num_heads * self.stored_dim, num_kv_heads * self.stored_dim, num_kv_heads * self.value_dim
+        blocks = {"q": stored_q}
         if own_kv:
-            self.add_child("qkv", Linear(hidden_size, self.q_size + 2 * self.kv_size,
-                                         parts={"q": self.q_size, "k": self.kv_size, "v": self.kv_size}))
-        else:
-            self.add_child("qkv", Linear(hidden_size, self.q_size, parts={"q": self.q_size}))
-        self.add_child("o", Linear(self.q_size, hidden_size))
+            blocks.update(k=stored_k, v=stored_v)
+        if head_gate:
+            blocks["g"] = num_heads
+        self.add_child("qkv", Linear(hidden_size, sum(blocks.values()), parts=blocks))
+        self.add_child("o", Linear(num_heads * self.value_dim, hidden_size))
+        rows = self.q_size + (2 * self.kv_size if own_kv else 0) + (num_heads if head_gate else 0)
+        self._relayout = self._relayout or rows % 8 != 0
+        self.gate_at = self.q_size + (2 * self.kv_size if own_kv else 0)      # first gate column of the kernels' rows
+        self._laid_out = False
         if qk_norm_eps is not None:
-            self.add_param("q_norm_weight", ParamSpec((head_dim,), init="norm", dtype="float32"))
+            self.add_param("q_norm_weight", ParamSpec((self.stored_dim,), init="norm", dtype="float32"))
             if own_kv:
-                self.add_param("k_norm_weight", ParamSpec((head_dim,), init="norm", dtype="float32"))
+                self.add_param("k_norm_weight", ParamSpec((self.stored_dim,), init="norm", dtype="float32"))
+        self.norm_eps = qk_norm_eps
         if position is not None:
             self.add_child("position", position)
         else:
@@ -55,10 +92,57 @@ class Attention(Mixer):
     def cache_need(self):
         return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
 
+    def set_param(self, local, tensor):
+        super().set_param(local, tensor)
+        self._laid_out = False
+
+    def finalize(self, device, dtype, max_positions):
+        """The kernels' layout of the stored parameters, where it differs (see the class text)."""
+        if not self._relayout or self._laid_out:
+            return
+        H, G, D, n, nv = self.num_heads, self.num_kv_heads, self.head_dim, self.stored_dim, self.value_dim
+        order = self.position.head_order() if self.position is not None and hasattr(self.position, "head_order") else None
+        take = torch.tensor(order if order is not None else list(range(n)) + [-1] * (D - n), dtype=torch.long)
+        w = self.qkv.weight
+        hidden = w.shape[1]
+
+        def heads(block, count, size, pick):
+            """[count * size, hidden] -> [count * D, hidden]: slot s of every head holds stored row pick[s] (zeros for -1)."""
+            wide = torch.cat((block.view(count, size, hidden), block.new_zeros(count, 1, hidden)), 1)
+            return wide[:, pick.to(block.device)].reshape(count * D, hidden)       # index -1 is the zero row
+
+        stored_q, stored_k = H * n, G * n
+        parts = [heads(w[:stored_q], H, n, take)]
+        at = stored_q
+        if self.own_kv:
+            keep = torch.tensor(list(range(nv)) + [-1] * (D - nv), dtype=torch.long)
+            parts += [heads(w[at:at + stored_k], G, n, take), heads(w[at + stored_k:at + stored_k + G * nv], G, nv, keep)]
+            at += stored_k + G * nv
+        if self.head_gate:
+            parts.append(w[at:at + H])
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts.append(w.new_zeros(8 - rows % 8, hidden))
+        self.qkv.weight = torch.cat(parts, 0).contiguous()
+        o = self.o.weight.view(-1, H, nv)
+        self.o.weight = torch.cat((o, o.new_zeros(o.shape[0], H, D - nv)), 2).reshape(-1, H * D).contiguous()
+        if self.norm_eps is not None:
+            # mean over D slots instead of n stored dimensions: eps and the weights take the ratio
+            self.qk_norm_eps = self.norm_eps * n / D
+            fix = math.sqrt(n / D)
+            for name in ("q_norm_weight", "k_norm_weight") if self.own_kv else ("q_norm_weight",):
+                wn = getattr(self, name)
+                wide = torch.cat((wn * fix, wn.new_zeros(1)))
+                setattr(self, name, wide[take.to(wn.device)].contiguous())
+        self._laid_out = True
+
     def forward(self, x, step, cache, state):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         grp = step.groups[cache.group]
-        qkv = self.qkv.forward(x)
+        packed = self.qkv.forward(x)
+        gated = self.head_gate
+        # the kernels' rows end where the gate columns (and the padding to whole steps of 8) begin
+        qkv = packed if packed.shape[1] == self.gate_at else packed[:, : self.gate_at]
         store = self.own_kv and cache.write
         qw = self.q_norm_weight if self.qk_norm_eps is not None else None
         kw = self.k_norm_weight if (self.qk_norm_eps is not None and self.own_kv) else qw
@@ -69,7 +153,9 @@ class Attention(Mixer):
             # only single tokens: norm, rotary, cache write and attention in one launch
             o = ops.decode_step_attention(qkv, qw, kw, eps, table, cache.k, cache.v, cache.page_size, grp.block_tables,
                                           step.context_lens, step.max_decode_context, self.scale, self.window,
-                                          Hq, Hkv, D, even_contexts=step.decode_contexts_even)
+                                          Hq, Hkv, D, even_contexts=step.decode_contexts_even, chunk=self.chunk)
+            if gated:
+                ops.head_gate(o, packed[:, self.gate_at:self.gate_at + Hq], Hq, D)
             return self.o.forward(o, allow_partials=True)
         if self.position is None or table is not None:
             # norm + rotary + cache write in one pass
@@ -78,7 +164,7 @@ class Attention(Mixer):
                 ops.qk_norm_rope_store(qkv, qw, kw, eps, table, step.positions, grp.slot_mapping,
                                        cache.k, cache.v, Hq, Hkv, D, cache.page_size, store=True, position_bound=bound)
             else:
-                rows = qkv if not self.own_kv else qkv[:, : self.q_size]
+                rows = qkv[:, : self.q_size]
                 ops.qk_norm_rope_store(rows, qw, kw, eps, table, step.positions, None, None, None,
                                        Hq, 0, D, cache.page_size, store=False, position_bound=bound)
         else:
@@ -91,12 +177,14 @@ class Attention(Mixer):
             k3 = qkv[:, self.q_size: self.q_size + nk * D].view(T, nk, D)
             self.position.apply(q3, k3, step.positions)
             if store:
-                v3 = qkv[:, self.q_size + self.kv_size:].view(T, Hkv, D)
+                v3 = qkv[:, self.q_size + self.kv_size: self.q_size + 2 * self.kv_size].view(T, Hkv, D)
                 ops.store_kv(k3, v3, grp.slot_mapping, cache.k, cache.v, cache.page_size)
         q = qkv[:, : self.q_size]
         o = ops.paged_attention(q, cache.k, cache.v, cache.page_size, grp.block_tables, step.context_lens,
                                 step.seq_of_token, step.positions, step.prefill_cu, step.num_decodes,
                                 step.max_decode_context, self.scale, self.window, Hq, Hkv, D,
                                 max_prefill_context=step.max_prefill_context,
-                                even_contexts=step.decode_contexts_even)
+                                even_contexts=step.decode_contexts_even, chunk=self.chunk)
+        if gated:
+            ops.head_gate(o, packed[:, self.gate_at:self.gate_at + Hq], Hq, D)
         return self.o.forward(o, allow_partials=True)

@@ -203,6 +203,15 @@ class PendingNorm:
         return self._new_residual
 
 
+class Settled:
+    """What a layer returns in place of its output when it has already added that output to the residual
+    stream (a block whose norms sit on the sublayers' outputs does): `rounded` is the stream in the compute
+    dtype, for the next layer's sublayers to read. Whoever comes next must not add anything to the residual."""
+
+    def __init__(self, rounded: torch.Tensor):
+        self.rounded = rounded
+
+
 class PositionEncoding(Part):
     """Something applied to queries and keys as a function of token positions."""
 

@@ -1,7 +1,7 @@
 """How norm, mixer and feed-forward are arranged in a layer (reference models/qwen3.py:55-74)."""
 from __future__ import annotations
 
-from .base import FeedForward, Mixer, Norm, Part, PendingNorm, register_part
+from .base import FeedForward, Mixer, Norm, Part, PendingNorm, Settled, register_part
 
 
 def norm_of(norm: Norm, x, residual):
@@ -36,6 +36,8 @@ class PreNormBlock(Part):
         return self.mixer.state_need()
 
     def forward(self, h, residual, step, cache, state):
+        if isinstance(h, Settled):          # the layer before has added its output already: the stream starts anew here
+            h, residual = residual, None
         # a part that takes it gets the norm before it as a `PendingNorm` and may run it inside its first product
         if getattr(self.mixer, "takes_pending_norm", False):
             x = PendingNorm(self.norm1, h, residual)
@@ -50,3 +52,42 @@ class PreNormBlock(Part):
             return out, x.new_residual()
         x, residual = norm_of(self.norm2, a, residual)
         return self.feed_forward.forward(x), residual
+
+
+@register_part("block", "output_norm")
+class OutputNormBlock(Part):
+    """stream += norm1(mixer(stream)); stream += norm2(feed_forward(stream)): the norms sit on the sublayers'
+    outputs only, and the sublayers read the stream itself (rounded to the compute dtype). Without a
+    feed-forward the layer is its first half. The stream is float32; each sum and each norm is one kernel
+    that also hands on the rounded stream."""
+
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm | None = None, feed_forward: FeedForward | None = None):
+        super().__init__()
+        if (norm2 is None) != (feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.add_child("norm1", norm1)
+        self.add_child("mixer", mixer)
+        if feed_forward is not None:
+            self.add_child("norm2", norm2)
+            self.add_child("feed_forward", feed_forward)
+        else:
+            self.norm2 = self.feed_forward = None
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def forward(self, h, residual, step, cache, state):
+        if isinstance(h, Settled):
+            x, stream = h.rounded, residual
+        elif residual is None:               # the first layer: the embedding's rows are the stream
+            x, stream = h, h.float()
+        else:                                # behind a layer that leaves its output to be added
+            stream = residual + (h.sum(0) if h.dim() == 3 else h).float()
+            x = stream.to(h.dtype if h.dim() == 2 else self.norm1.out_dtype)
+        x, stream = self.norm1.add_to(self.mixer.forward(x, step, cache, state), stream)
+        if self.feed_forward is not None:
+            x, stream = self.norm2.add_to(self.feed_forward.forward(x), stream)
+        return Settled(x), stream

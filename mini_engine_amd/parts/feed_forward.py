@@ -29,3 +29,19 @@ class SwiGLU(FeedForward):
             return self.down.forward(self.gate_up.forward(x, gated=True), allow_partials=True)
         gu = self.gate_up.forward(x)
         return ops.silu_mul_linear(gu, self.down.weight, allow_partials=True)
+
+
+@register_part("feed_forward", "dense")
+class ActivatedMLP(FeedForward):
+    """down(act(up(x))) without a gate; `activation`: "relu2" (the square of relu) or "silu"."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2"):
+        super().__init__()
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(ops.ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.add_child("up", Linear(hidden_size, intermediate_size))
+        self.add_child("down", Linear(intermediate_size, hidden_size))
+
+    def forward(self, x):
+        return self.down.forward(ops.activation(self.up.forward(x), self.activation), allow_partials=True)

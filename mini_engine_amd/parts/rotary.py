@@ -16,23 +16,58 @@ class RotaryEmbedding(PositionEncoding):
     (cos, sin) adjacent, the form the fused query/key kernel reads.
     """
 
-    def __init__(self, head_dim: int, theta: float):
+    def __init__(self, head_dim: int, theta: float, rotary_dims: int | None = None, interleaved: bool = False,
+                 stored_dim: int | None = None, exact_angles: bool = False):
+        """`rotary_dims`: only the first so many of a head's `stored_dim` dimensions turn, with angles
+        p * theta^(-2i/rotary_dims); the others pass unchanged (None: all `head_dim` turn). `interleaved`: the
+        stored pairs are (x_2i, x_2i+1) instead of (x_i, x_i+rotary_dims/2). Either way the kernels see the
+        half-split form over `head_dim` slots (which may exceed `stored_dim`: slots that hold nothing): a mixer
+        lays its query and key heads out by `head_order()`, which puts the two members of pair i into slots i and
+        head_dim/2 + i, the dimensions that do not turn into the slots left, whose table entries are (cos, sin)
+        = (1, 0). A dot product does not care about the order of the dimensions as long as q and k share it."""
         super().__init__()
         if head_dim % 2:
             raise ValueError("rotary encoding needs an even head size")
         self.head_dim = head_dim
         self.theta = float(theta)
+        self.stored_dim = head_dim if stored_dim is None else int(stored_dim)
+        self.rotary_dims = self.stored_dim if rotary_dims is None else int(rotary_dims)
+        self.interleaved = bool(interleaved)
+        self.exact_angles = bool(exact_angles)     # angles, cos and sin formed in float64 and rounded once to float32
+        if self.rotary_dims % 2 or not 0 <= self.rotary_dims <= self.stored_dim <= head_dim:
+            raise ValueError(f"{self.rotary_dims} rotating dimensions of {self.stored_dim} stored in {head_dim} slots")
         self.table = None
+
+    def head_order(self) -> list | None:
+        """Which stored dimension of a head each of the `head_dim` slots holds (-1: none, the slot is zero); None
+        when the stored order is the kernels' order already."""
+        D, n, r = self.head_dim, self.stored_dim, self.rotary_dims
+        if n == D and r == D and not self.interleaved:
+            return None
+        if self.interleaved:
+            low, high = [2 * i for i in range(r // 2)], [2 * i + 1 for i in range(r // 2)]
+        else:
+            low, high = list(range(r // 2)), list(range(r // 2, r))
+        rest = list(range(r, n))
+        room = D // 2 - r // 2
+        low, high = low + rest[:room], high + rest[room:]
+        return low + [-1] * (D // 2 - len(low)) + high + [-1] * (D // 2 - len(high))
 
     def finalize(self, device, dtype, max_positions):
         if self.table is not None and self.table.shape[0] >= max_positions and self.table.device == torch.device(device):
             return
         half = self.head_dim // 2
         # same expression as the reference: 1 / theta^(2i/D), float32 throughout
-        inv_freq = 1.0 / (self.theta ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim))
+        turning = self.rotary_dims
+        inv_freq = 1.0 / (self.theta ** (torch.arange(0, turning, 2, dtype=torch.float32) / max(turning, 1)))
         t = torch.arange(max_positions, dtype=torch.float32)
-        ang = torch.outer(t, inv_freq)                      # [P, D/2]
-        self.table = torch.stack((ang.cos(), ang.sin()), dim=-1).contiguous().to(device)
+        ang = torch.zeros((max_positions, half), dtype=torch.float32)
+        ang[:, :turning // 2] = torch.outer(t, inv_freq)    # [P, D/2]; angle 0 where nothing turns
+        if self.exact_angles:
+            ang = ang.double()
+            rate = self.theta ** (-torch.arange(0, turning, 2, dtype=torch.float64) / max(turning, 1))
+            ang[:, :turning // 2] = torch.outer(torch.arange(max_positions, dtype=torch.float64), rate)
+        self.table = torch.stack((ang.cos(), ang.sin()), dim=-1).float().contiguous().to(device)
         assert self.table.shape == (max_positions, half, 2)
 
     def rotary_table(self):

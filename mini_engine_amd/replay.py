@@ -24,7 +24,7 @@ ROUND = 64     # a request's token count is rounded up to this (or to the page s
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda",
-                 poison_cache: bool = False):
+                 poison_cache: bool = False, state_slots: int = 4):
         if dtype not in DTYPES:
             raise ValueError(f"--dtype must be one of {sorted(DTYPES)}")
         if page_size > ROUND and page_size % ROUND:
@@ -37,7 +37,7 @@ class Replayer:
         self.max_positions = max_tokens if limit is None else min(max_tokens, limit)
         self.model = load_model(model_dir, device, DTYPES[dtype], self.max_positions, cfg)
         plan = self.model.cache_plan()
-        slots = 8 if any(s is not None for s in plan.state_needs) else 0
+        slots = state_slots if any(s is not None for s in plan.state_needs) else 0
         self.manager = CacheManager(max_tokens // page_size, page_size, ModelRunner.windows_of(self.model),
                                     num_state_slots=slots, enable_prefix_caching=False)
         self.runner = ModelRunner(self.model, self.manager, DTYPES[dtype], device, self.max_positions,
@@ -74,10 +74,12 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at a time (each rounded up to a multiple of 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--state-slots", type=int, default=4, help="requests that can be live at a time in a model that keeps "
+                    "per-request state (their slots are used again as requests end)")
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     print(f"[trace_run] loading {args.model} ({args.dtype}); kernels are compiled on first use", file=sys.stderr, flush=True)
-    rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size)
+    rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size, state_slots=args.state_slots)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     for line in sys.stdin:
         line = line.strip()

@@ -82,7 +82,8 @@ def store_kv(k, v, slots, k_cache, v_cache, page):
 
 def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_of_token, positions,
                     prefill_cu, num_decodes, max_decode_context, scale, window, Hq, Hkv, D,
-                    force_simple=False, max_prefill_context=0, even_contexts=False, compute_dtype=torch.float32):
+                    force_simple=False, max_prefill_context=0, even_contexts=False, compute_dtype=torch.float32,
+                    chunk=None, decode_as_prefill=False):
     """Token by token: gather the keys this token may see through its request's block table
     and nothing else (so unowned pages are never read), softmax, weighted sum."""
     T = q.shape[0]
@@ -92,6 +93,8 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
     for t in range(T):
         b, pos = seqs[t], where[t]
         lo = max(0, pos - window + 1) if window else 0
+        if chunk:
+            lo = pos - pos % chunk                         # a block mask: only the keys of the query's own block
         hi = min(pos + 1, lens[b])                         # a padding row (context 0) sees nothing
         if hi <= lo:
             out[t] = 0
@@ -110,7 +113,8 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
 
 
 def decode_step_attention(qkv, q_weight, k_weight, eps, table, k_cache, v_cache, page, block_tables, context_lens,
-                          max_context, scale, window, Hq, Hkv, D, even_contexts=False, compute_dtype=torch.float32):
+                          max_context, scale, window, Hq, Hkv, D, even_contexts=False, compute_dtype=torch.float32,
+                          chunk=None):
     """The two twins above, one after the other, on a copy of the rows: row r is request r's new token at
     position context_lens[r] - 1, its slot is what the block table names for that position (a row with
     context 0 is padding: nothing is written for it and it sees nothing)."""
@@ -124,7 +128,7 @@ def decode_step_attention(qkv, q_weight, k_weight, eps, table, k_cache, v_cache,
     qk_norm_rope_store(rows, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache, Hq, Hkv, D, page, store=True)
     seq = torch.arange(B, dtype=torch.int32, device=qkv.device)
     return paged_attention(rows[:, :Hq * D], k_cache, v_cache, page, block_tables, context_lens, seq, positions, None, B,
-                           max_context, scale, window, Hq, Hkv, D, compute_dtype=compute_dtype)
+                           max_context, scale, window, Hq, Hkv, D, compute_dtype=compute_dtype, chunk=chunk)
 
 
 def linear(x, w, out_dtype=None, allow_partials=False, out=None):
@@ -159,6 +163,92 @@ def norm_linear(x, residual, norm_weight, eps, w, out_dtype=None, want_residual=
 
 def silu_mul_linear(gu, w, allow_partials=False):
     return linear(silu_and_mul(gu), w)
+
+
+def add_rms_norm(y, weight, eps, stream, out_dtype):
+    """stream + weight * y / rms(y) in float32 -> (rounded to out_dtype, float32)."""
+    r = y.float().sum(0) if y.dim() == 3 else y.float()
+    new = stream + weight * (r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps))
+    return (new if out_dtype == torch.float32 else new.to(out_dtype)), new
+
+
+def activation(x, kind):
+    v = x.float()
+    v = v * torch.sigmoid(v) if kind == "silu" else torch.relu(v) ** 2
+    return v.to(x.dtype)
+
+
+def head_gate(o, gate, H, D):
+    T = o.shape[0]
+    o.copy_((o.float().view(T, H, D) * torch.sigmoid(gate.float())[:, :, None]).view(T, H * D).to(o.dtype))
+
+
+def causal_conv(x, weight, bias, state, state_slots, cu_seqlens, seq_of_token):
+    """x [T, C]; weight float32 [C, taps] (the last tap is the current token's), bias [C]; state [slots, C * (taps - 1)]
+    float32: per channel the inputs before the request's next token, oldest first. silu(conv) in x's dtype; the state
+    moves on."""
+    T, C = x.shape
+    taps = weight.shape[1]
+    out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    cu, slots = cu_seqlens.tolist(), state_slots.tolist()
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi <= lo:
+            continue
+        held = state[slots[b]].view(C, taps - 1).t()                  # [taps - 1, C]
+        seen = torch.cat((held, x[lo:hi].float()), 0)                  # [taps - 1 + n, C]
+        acc = bias.float().expand(hi - lo, C).clone()
+        for j in range(taps):
+            acc += weight[:, j].float() * seen[j:j + hi - lo]
+        out[lo:hi] = (acc * torch.sigmoid(acc)).to(x.dtype)
+        state[slots[b]] = seen[seen.shape[0] - (taps - 1):].t().reshape(-1)
+    return out
+
+
+def softplus(x):
+    return torch.where(x > 20, x, torch.log1p(torch.exp(torch.clamp(x, max=20))))
+
+
+def linear_recurrence(q, k, v, state, state_slots, cu_seqlens, q_lens, H, G, N, P, decay=None, dt=None, dt_bias=None,
+                      rate=None, skip=None):
+    """S_t = a S_(t-1) + b k_t v_t^T, y_t = S_t^T q_t (+ skip v_t), float32, token by token. q, k [T, G * N], v [T, H * P];
+    state [slots, H * N * P]. a, b: decay[h], 1; or exp(-rate[h] dt), dt with dt = softplus(dt[t, h] + dt_bias[h])."""
+    T = v.shape[0]
+    y = torch.zeros((T, H * P), dtype=torch.float32, device=v.device)
+    cu, slots = cu_seqlens.tolist(), state_slots.tolist()
+    per = H // G
+    for b in range(len(cu) - 1):
+        S = state[slots[b]].view(H, N, P).clone()
+        for t in range(cu[b], cu[b + 1]):
+            kt, qt, vt = k[t].float().view(G, N), q[t].float().view(G, N), v[t].float().view(H, P)
+            if decay is not None:
+                a, bb = decay.float(), torch.ones(H)
+            else:
+                step = softplus(dt[t].float() + dt_bias)
+                a, bb = torch.exp(-rate * step), step
+            kh, qh = kt.repeat_interleave(per, 0), qt.repeat_interleave(per, 0)
+            S = a[:, None, None] * S + (bb[:, None] * kh)[:, :, None] * vt[:, None, :]
+            out = torch.einsum("hnp,hn->hp", S, qh)
+            if skip is not None:
+                out = out + skip[:, None] * vt
+            y[t] = out.reshape(-1)
+        state[slots[b]] = S.reshape(-1)
+    return y
+
+
+def gated_rms_norm(y, gate, weight, eps, groups, kind, out_dtype):
+    """kind "silu_before": unit rms per group of (y * silu(gate)), times weight; "sigmoid_behind": unit rms of y, times
+    weight, times sigmoid(gate). y float32 [T, n] or partial sums [S, T, n]."""
+    r = y.float().sum(0) if y.dim() == 3 else y.float()
+    g = gate.float()
+    T, n = r.shape
+    if kind == "silu_before":
+        r = r * (g * torch.sigmoid(g))
+    r = r.view(T, groups, n // groups)
+    r = (r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * weight
+    if kind == "sigmoid_behind":
+        r = r * torch.sigmoid(g)
+    return r.to(out_dtype)
 
 
 def _fmix32(h):
@@ -228,3 +318,9 @@ class PlainBackend:
     norm_linear = staticmethod(norm_linear)
     gated_linear = staticmethod(gated_linear)
     sample = staticmethod(sample)
+    add_rms_norm = staticmethod(add_rms_norm)
+    activation = staticmethod(activation)
+    head_gate = staticmethod(head_gate)
+    causal_conv = staticmethod(causal_conv)
+    linear_recurrence = staticmethod(linear_recurrence)
+    gated_rms_norm = staticmethod(gated_rms_norm)
