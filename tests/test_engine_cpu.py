@@ -235,7 +235,7 @@ def test_replay_program_on_cpu(folders, plain_backend, tmp_path, monkeypatch, ca
     ]
     monkeypatch.setattr("sys.stdin", io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"))
     real = replay.Replayer
-    monkeypatch.setattr(replay, "Replayer", lambda m, d, n, p: real(m, d, n, p, device="cpu", poison_cache=True))
+    monkeypatch.setattr(replay, "Replayer", lambda m, d, n, p, **kw: real(m, d, n, p, device="cpu", poison_cache=True, **kw))
     assert replay.main(["--model", folder, "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "128",
                         "--page-size", "8"]) == 0
     assert capsys.readouterr().out.split("\n")[:4] == ["done 0", "done 1", "done 2", "done 3"]

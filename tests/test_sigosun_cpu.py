@@ -1,0 +1,103 @@
+"""Sigosun on the CPU: configuration, checkpoint layout, and the engine's bookkeeping for it (pages, state slots,
+batches, cuts, the scheduler) with the plain twins of the kernels in float32, against the plain evaluation."""
+import json
+import os
+
+import pytest
+import torch
+
+import sigosun_cases as S
+from mini_engine_amd.cache.manager import CacheManager
+from mini_engine_amd.config.model_config import ConfigError, SigosunConfig, load_model_config
+from mini_engine_amd.engine.runner import ModelRunner
+from mini_engine_amd.parts.rotary import RotaryEmbedding
+from mini_engine_amd.registry import build_model
+from mini_engine_amd.weights.loader import load_model
+
+
+@pytest.fixture(scope="module")
+def sigosun_folders(tmp_path_factory):
+    made = {}
+
+    def get(name):
+        if name not in made:
+            made[name] = S.make_folder(name, str(tmp_path_factory.mktemp(f"sigosun_{name}")))
+        return made[name]
+
+    return get
+
+
+class Env:
+    device, dtype, tol = "cpu", torch.float32, 2e-5
+
+    def __init__(self, folders):
+        self.folders, self.models = folders, {}
+
+    def runner(self, name, pages, slots):
+        folder = self.folders(name)
+        if name not in self.models:
+            self.models[name] = load_model(folder, self.device, self.dtype, 512)
+        model = self.models[name]
+        manager = CacheManager(pages, S.PAGE[name], ModelRunner.windows_of(model), num_state_slots=slots, enable_prefix_caching=False)
+        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True), manager, folder
+
+
+def test_config_reads_back_and_refuses_what_it_cannot_run(tmp_path):
+    for name, raw in S.CONFIGS.items():
+        cfg = SigosunConfig.from_dict(raw)
+        assert SigosunConfig.from_dict(cfg.to_dict()) == cfg
+        assert len(cfg.layers) == len(raw["layers"]) and cfg.vocab_size == raw["vocab"]
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(S.CONFIGS["mix"], f)
+    assert isinstance(load_model_config(str(tmp_path)), SigosunConfig)          # chosen by the file's architecture name
+    bad = json.loads(json.dumps(S.CONFIGS["mix"]))
+    bad["layers"][3]["mixer"]["kv_from"] = 2                                    # not an attention layer
+    with pytest.raises(ConfigError):
+        SigosunConfig.from_dict(bad)
+    bad = json.loads(json.dumps(S.CONFIGS["mix"]))
+    bad["layers"][2]["mixer"]["decay"] = [0.5]
+    with pytest.raises(ConfigError):
+        SigosunConfig.from_dict(bad)
+    bad = json.loads(json.dumps(S.CONFIGS["mix"]))
+    del bad["layers"][0]["mixer"]["state"]
+    with pytest.raises(ConfigError, match="state"):
+        SigosunConfig.from_dict(bad)
+
+
+def test_model_is_assembled_from_the_config():
+    model = build_model(SigosunConfig.from_dict(S.CONFIGS["mix"]))
+    plan = model.cache_plan()
+    assert plan.call_group == [None, 0, None, 0, None] and plan.call_writes == [False, True, False, False, False]
+    assert [s is not None for s in plan.state_needs] == [True, False, True, False, True]
+    assert plan.state_needs[0].shape == (4 * 20 * 12 + (48 + 2 * 2 * 20) * 3,)       # matrices, then the convolution's inputs
+    names = {src.name for sources in model.weight_sources.values() for src in sources}
+    assert {"embed", "head", "final.norm", "l0.mix.in", "l0.mix.conv.b", "l1.mix.k.norm", "l1.mix.g", "l2.mix.norm", "l3.mix.q",
+            "l0.mlp.up", "l1.norm2"} <= names
+    assert not any(n.startswith("l3.mix.k") or n.startswith("l3.mix.v") or n.startswith("l2.mlp") for n in names)
+
+
+def test_head_order_of_rotations():
+    assert RotaryEmbedding(16, 1e4).head_order() is None
+    assert RotaryEmbedding(8, 1e4, interleaved=True).head_order() == [0, 2, 4, 6, 1, 3, 5, 7]
+    # 4 of 10 stored dimensions turn, in 16 slots: the pairs half a head apart, the rest behind them, empty slots last
+    order = RotaryEmbedding(16, 1e4, rotary_dims=4, interleaved=True, stored_dim=10).head_order()
+    assert order == [0, 2, 4, 5, 6, 7, 8, 9, 1, 3, -1, -1, -1, -1, -1, -1]
+    r = RotaryEmbedding(16, 100.0, rotary_dims=4, interleaved=True, stored_dim=10, exact_angles=True)
+    r.finalize("cpu", torch.float32, 8)
+    assert torch.equal(r.table[:, 2:, 0], torch.ones(8, 6)) and torch.equal(r.table[:, 2:, 1], torch.zeros(8, 6))
+    assert abs(float(r.table[3, 1, 1]) - float(torch.sin(torch.tensor(3 * 100.0 ** -0.5, dtype=torch.float64)))) < 1e-7
+
+
+@pytest.mark.parametrize("name", ["mix", "att", "ssm", "lin"])
+@pytest.mark.parametrize("case", S.ALL, ids=lambda c: c.__name__)
+def test_cuts(sigosun_folders, plain_backend, case, name):
+    case(Env(sigosun_folders), name)
+
+
+def test_far_keys_and_block_edges(sigosun_folders, plain_backend):
+    S.far_keys(Env(sigosun_folders))
+
+
+@pytest.mark.parametrize("name", ["mix", "lin"])
+def test_greedy_generation_through_the_scheduler(sigosun_folders, plain_backend, name):
+    S.greedy_through_the_engine("cpu", "float32", name, sigosun_folders(name), exact=True)
