@@ -37,7 +37,7 @@ import time
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-from mini_engine_amd.config.sizes import SIZES, model_config   # noqa: E402  (the named layer sizes)
+from mini_engine_amd.config.sizes import SIZES, model_config, sigosun_config   # noqa: E402  (the named layer sizes)
 
 
 def log(msg: str) -> None:
@@ -97,7 +97,20 @@ def decode_bytes(model, item: int, contexts: list, page: int, dtype) -> int:
     kv = 0.0
     for per_token, window in cache_bytes_per_token(model, page, dtype):
         kv += per_token * sum(min(c, window) if window else c for c in contexts)
-    return int(weights + kv)
+    for call in model.order:                      # a block mask bounds what a request reads as a window does
+        mixer = getattr(model.layers[call.layer], "mixer", None)
+        chunk = getattr(mixer, "chunk", None)
+        if chunk:
+            per_token = 2 * mixer.num_kv_heads * mixer.head_dim * item
+            kv -= per_token * sum(c - ((c - 1) % chunk + 1) for c in contexts)
+    state = 0
+    for need in model.cache_plan().state_needs:   # a request's state is read and written once a step
+        if need is not None:
+            n = 1
+            for d in need.shape:
+                n *= int(d)
+            state += 2 * 4 * n * len(contexts)
+    return int(weights + kv + state)
 
 
 def prefill_flops(model, T: int) -> float:
@@ -110,9 +123,15 @@ def prefill_flops(model, T: int) -> float:
         mixer = getattr(model.layers[call.layer], "mixer", None)
         heads, size = getattr(mixer, "num_heads", None), getattr(mixer, "head_dim", None)
         if heads and size:
-            window = getattr(mixer, "window", None)
+            window, chunk = getattr(mixer, "window", None), getattr(mixer, "chunk", None)
             seen = sum(min(t + 1, window) if window else t + 1 for t in range(T)) if window else T * (T + 1) / 2
+            if chunk:
+                seen = sum(t % chunk + 1 for t in range(T))
             attn += 4.0 * heads * size * seen
+        elif heads and hasattr(mixer, "state_need"):
+            # a state of N x P per head: one multiply-add to move it on and one to read it, per token
+            rows = getattr(mixer, "state_dim", None) or getattr(mixer, "key_dim", 0)
+            attn += 4.0 * heads * rows * mixer.value_dim * T
     return 2.0 * T * per_token + attn + 2.0 * head
 
 
@@ -301,12 +320,14 @@ def resolve_model(args, size: str, layers, tmp: str) -> tuple:
         if checkpoint_files(size):
             return cfg, full, label, size, None, "the folder's checkpoint"
         return cfg, full, label, size, args.seed, "drawn on the device"
-    cfg, full = model_config(size, layers)
+    design = size.startswith("sigosun:")
+    cfg, full = sigosun_config(size.split(":")[1], layers) if design else model_config(size, layers)
     skeleton = build_model(cfg)                              # declared parameters only, no tensors
     params = sum(_spec_bytes(spec, 1) for _, _, _, spec in skeleton.named_specs())
     on_device = args.weights == "device" or (args.weights == "auto" and params > 2e9)
-    folder, random_weights = folder_for(cfg, args.seed, os.path.join(tmp, size), on_device)
-    return cfg, full, f"Qwen3-{size} sizes", folder, random_weights, "drawn on the device" if on_device else "written folder"
+    folder, random_weights = folder_for(cfg, args.seed, os.path.join(tmp, size.replace(":", "_")), on_device)
+    label = f"Sigosun at the Qwen3-{size.split(':')[1]} layer sizes" if design else f"Qwen3-{size} sizes"
+    return cfg, full, label, folder, random_weights, "drawn on the device" if on_device else "written folder"
 
 
 def describe(cfg, label: str, full_layers) -> dict:
@@ -377,6 +398,26 @@ def other_size(run: dict, context: int) -> dict:
     return obj
 
 
+def design_comparison(args) -> int:
+    """`--design`: the design and Qwen3 side by side at each named size, one JSON line."""
+    points = [int(p) for p in args.points.split(",") if p and int(p) != args.batch]
+    steps, warmup = min(args.steps, 32), min(args.warmup, 4)
+    rows = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        for size in [s for s in args.design_sizes.split(",") if s]:
+            pair = {}
+            for name, which in ((args.design, f"{args.design}:{size}"), ("qwen3", size)):
+                run = measure(args, which, args.layers, tmp, [args.batch] + points, steps, warmup)
+                pair[name] = other_size(run, args.context)
+            rows[size] = pair
+    line = {"metric": f"{args.design} beside qwen3: prefill tok/s at {args.prefill_tokens} tokens, decode tok/s at batch "
+                      f"{args.batch}/{'/'.join(map(str, points))}", "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: seeded random token ids and weights",
+            "sizes": rows}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -411,7 +452,13 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
+    ap.add_argument("--design", default=None, choices=["sigosun"],
+                    help="instead of the default workload: prefill and decode throughput of this design at the layer sizes "
+                         "named by --design-sizes (random weights), each beside Qwen3 at the same width, depth and vocabulary")
+    ap.add_argument("--design-sizes", default="0.6b,8b")
     args = ap.parse_args(argv)
+    if args.design:
+        return design_comparison(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2

@@ -269,6 +269,10 @@ class SigosunConfig:
     eos_token_id: int | None = None
     max_position_embeddings: int | None = None
 
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
     MIXER_KEYS = {
         "attention": (("heads", int), ("kv_heads", int), ("dim", int), ("vdim", int), ("scale", float)),
         "mamba2": (("heads", int), ("vdim", int), ("state", int), ("groups", int), ("conv", int), ("norm_groups", int)),

@@ -3,7 +3,7 @@ with random weights (no model folder at hand). The figures are those of the publ
 files; a model folder's own config.json always wins where there is one."""
 from __future__ import annotations
 
-from .model_config import Qwen3Config
+from .model_config import Qwen3Config, SigosunConfig
 
 SIZES = {
     # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
@@ -24,3 +24,36 @@ def model_config(size: str, layers: int | None = None):
         architectures=["Qwen3ForCausalLM"], vocab_size=V, hidden_size=h, intermediate_size=I,
         num_hidden_layers=layers or L, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
         rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=tied, max_position_embeddings=40960)), L
+
+
+def sigosun_config(size: str, layers: int | None = None):
+    """(a Sigosun configuration whose layers resemble that size's: the same width, vocabulary, feed-forward width and
+    attention heads, with `layers` layers or as many as the size has; that count). The mixers take turns: linear
+    attention, attention with keys of its own, a state-space layer, linear attention, attention on the keys of the
+    attention layer before it, a state-space layer; the attention layers carry the feed-forwards. Blocks of 2,048
+    positions, half of each head's dimensions turning; state-space heads of 64 with a state of 128; linear
+    attention with the attention layers' head size."""
+    L, h, Hq, Hkv, D, I, V, _ = SIZES[size]
+    n = layers or L
+    attention = lambda src: {"type": "attention", "mlp": {"kind": "dense", "ff": I},
+                             "mixer": dict({"heads": Hq, "kv_heads": Hkv, "dim": D, "vdim": D, "scale": D ** -0.5,
+                                            "rot": {"dims": D // 2, "base": 1e6}, "mask": {"size": 2048}},
+                                           **({} if src is None else {"kv_from": src}))}
+    space = {"type": "mamba2", "mlp": None, "mixer": {"heads": 2 * h // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4,
+                                                      "norm_groups": 1}}
+    linear = {"type": "lightning", "mlp": None,
+              "mixer": {"heads": Hq, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5 - 8 * i / max(1, Hq - 1)) for i in range(Hq)]}}
+    out, last_own = [], None
+    for i in range(n):
+        turn = i % 6
+        if turn in (0, 3):
+            out.append(linear)
+        elif turn in (2, 5):
+            out.append(space)
+        elif turn == 1 or last_own is None:
+            out.append(attention(None))
+            last_own = i
+        else:
+            out.append(attention(last_own))
+    return SigosunConfig.from_dict({"architecture": "Sigosun", "vocab": V, "width": h, "norm": {"eps": 1e-6}, "layers": out,
+                                    "max_position_embeddings": 40960}), L

@@ -59,7 +59,7 @@ CONFIGS = {
     ]),
     # each mechanism alone
     "att": _model(64, 32, 1e-6, [_att(6, 2, 16, 16, 0.25, 16, 10000.0, 5, ff=48)]),
-    "ssm": _model(64, 40, 1e-5, [_ssm(3, 80, 70, 1, 3, 1)]),          # value size above 64, state above 64 rows
+    "ssm": _model(64, 36, 1e-5, [_ssm(3, 80, 70, 1, 3, 1)]),          # value size above 64, state above 64 rows, a width that is no multiple of 8
     "lin": _model(64, 24, 1e-5, [_lin(2, 72, 8, [0.8, 0.9995])]),     # key size above 64: two slices of the state
     # long blocks: keys far back among hundreds; 1 key head for 3 query heads; key size 32 against value size 16
     "far": _model(80, 32, 1e-5, [_att(3, 1, 32, 16, 0.2, 32, 250000.0, 300, ff=40), _lin(1, 16, 16, [0.999]),
