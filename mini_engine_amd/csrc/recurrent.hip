@@ -39,20 +39,64 @@ __global__ void add_rms_norm_kernel(const TX* __restrict__ y, int parts, int64_t
   }
 }
 
+// The same with every operand of a row asked for at once and kept in registers (rows of up to BD * 8 elements): one
+// trip to memory before the workgroup's sum and none behind it, which is what a step of a few rows waits for.
+template <typename TX, typename TY>
+__global__ void add_rms_norm_regs_kernel(const TX* __restrict__ y, int parts, int64_t part_stride, const float* __restrict__ w,
+                                         const float* __restrict__ stream_in, float* __restrict__ stream_out,
+                                         TY* __restrict__ rounded, int n, float eps) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const TX* yr = y + t * n;
+  float yv[8], sv[8], wv[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    yv[k] = 0.f; sv[k] = 0.f; wv[k] = 0.f;
+    if (i < n) {
+      for (int p = 0; p < parts; ++p) yv[k] += to_f32<TX>(yr[p * part_stride + i]);
+      sv[k] = stream_in[t * n + i];
+      wv[k] = w[i];
+    }
+    ss += yv[k] * yv[k];
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i < n) {
+      const float r = sv[k] + yv[k] * inv * wv[k];
+      stream_out[t * n + i] = r;
+      if (rounded) rounded[t * n + i] = from_f32<TY>(r);
+    }
+  }
+}
+
+template <typename TX, typename TY>
+static void launch_add_rms_norm(const TX* y, int parts, int64_t part_stride, const float* w, const float* stream_in,
+                                float* stream_out, TY* rounded, int64_t T, int n, float eps, hipStream_t stream) {
+  if (n <= 8192) {
+    const int threads = n <= 512 ? 64 : (n <= 2048 ? 256 : 1024);
+    add_rms_norm_regs_kernel<TX, TY><<<dim3((unsigned)T), dim3(threads), 0, stream>>>(y, parts, part_stride, w, stream_in,
+                                                                                     stream_out, rounded, n, eps);
+    return;
+  }
+  add_rms_norm_kernel<TX, TY><<<dim3((unsigned)T), dim3(256), (size_t)n * sizeof(float), stream>>>(y, parts, part_stride, w, stream_in,
+                                                                                                 stream_out, rounded, n, eps);
+}
+
 extern "C" int me_add_rms_norm(const void* y, int y_dtype, int parts, int64_t part_stride, const float* w,
                                const float* stream_in, float* stream_out, void* rounded, int64_t T, int n, float eps,
                                hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(n >= 1 && n <= 15360, "add_rms_norm: width %d outside 1..15360", n);
   ME_CHECK(parts >= 1 && parts <= RC_MAX_PARTIALS && (parts == 1 || y_dtype == ME_F32), "add_rms_norm: up to %d float32 partial sums", RC_MAX_PARTIALS);
-  const dim3 grid((unsigned)T), block(n >= 1024 ? 256 : (n > 256 ? 128 : 64));
-  const size_t lds = (size_t)n * sizeof(float);
   if (y_dtype == ME_F32)
-    add_rms_norm_kernel<float, float><<<grid, block, lds, stream>>>((const float*)y, parts, part_stride, w, stream_in, stream_out,
-                                                                    (float*)nullptr, n, eps);
+    launch_add_rms_norm<float, float>((const float*)y, parts, part_stride, w, stream_in, stream_out, (float*)nullptr, T, n, eps, stream);
   else
-    add_rms_norm_kernel<bf16_t, bf16_t><<<grid, block, lds, stream>>>((const bf16_t*)y, parts, part_stride, w, stream_in,
-                                                                      stream_out, (bf16_t*)rounded, n, eps);
+    launch_add_rms_norm<bf16_t, bf16_t>((const bf16_t*)y, parts, part_stride, w, stream_in, stream_out, (bf16_t*)rounded, T, n, eps, stream);
   ME_LAUNCH_CHECK();
   return 0;
 }
@@ -63,9 +107,7 @@ extern "C" int me_add_rms_norm_partials(const float* y, int parts, int64_t part_
   if (T == 0) return 0;
   ME_CHECK(n >= 1 && n <= 15360, "add_rms_norm: width %d outside 1..15360", n);
   ME_CHECK(parts >= 1 && parts <= RC_MAX_PARTIALS, "add_rms_norm: up to %d partial sums", RC_MAX_PARTIALS);
-  const dim3 grid((unsigned)T), block(n >= 1024 ? 256 : (n > 256 ? 128 : 64));
-  add_rms_norm_kernel<float, bf16_t><<<grid, block, (size_t)n * sizeof(float), stream>>>(y, parts, part_stride, w, stream_in,
-                                                                                        stream_out, (bf16_t*)rounded, n, eps);
+  launch_add_rms_norm<float, bf16_t>(y, parts, part_stride, w, stream_in, stream_out, (bf16_t*)rounded, T, n, eps, stream);
   ME_LAUNCH_CHECK();
   return 0;
 }
@@ -168,6 +210,25 @@ __global__ void causal_conv_state_kernel(const TX* __restrict__ x, int64_t x_str
   for (int s = 0; s < taps - 1; ++s) held[s] = next[s];
 }
 
+// A step of single tokens (token b is request b's): output and state in one pass, one thread per (request, channel).
+template <typename TX>
+__global__ void causal_conv_step_kernel(const TX* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                                        const float* __restrict__ bias, float* __restrict__ state, int64_t state_stride,
+                                        const int32_t* __restrict__ slots, TX* __restrict__ out, int C, int taps) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  float* held = state + (int64_t)slots[b] * state_stride + (int64_t)c * (taps - 1);
+  const float now = to_f32<TX>(x[(int64_t)b * x_stride + c]);
+  float seen[CONV_MAX_TAPS];
+  for (int s = 0; s < taps - 1; ++s) seen[s] = held[s];
+  float acc = bias[c] + w[(int64_t)c * taps + taps - 1] * now;
+  for (int s = 0; s < taps - 1; ++s) acc += w[(int64_t)c * taps + s] * seen[s];
+  out[(int64_t)b * C + c] = from_f32<TX>(silu_f(acc));
+  for (int s = 0; s + 1 < taps - 1; ++s) held[s] = seen[s + 1];
+  if (taps > 1) held[taps - 2] = now;
+}
+
 extern "C" int me_causal_conv(const void* x, int64_t x_stride, int dtype, const float* w, const float* bias, float* state,
                               int64_t state_stride, const int32_t* slots, const int32_t* cu, const int32_t* seq_of_token,
                               void* out, int64_t T, int num_seqs, int C, int taps, hipStream_t stream) {
@@ -177,6 +238,16 @@ extern "C" int me_causal_conv(const void* x, int64_t x_stride, int dtype, const 
   ME_CHECK(T <= 2147483647ll && num_seqs <= 65535 && (C + block.x - 1) / block.x <= 65535,
            "causal_conv: too many tokens, requests or channels for one launch");
   const dim3 grid((unsigned)T, (C + block.x - 1) / block.x);
+  if (T == num_seqs) {                     // every request brings one token
+    if (dtype == ME_F32)
+      causal_conv_step_kernel<float><<<grid, block, 0, stream>>>((const float*)x, x_stride, w, bias, state, state_stride, slots,
+                                                                 (float*)out, C, taps);
+    else
+      causal_conv_step_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, x_stride, w, bias, state, state_stride, slots,
+                                                                  (bf16_t*)out, C, taps);
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == ME_F32)
     causal_conv_kernel<float><<<grid, block, 0, stream>>>((const float*)x, x_stride, w, bias, state, state_stride, slots, cu,
                                                           seq_of_token, (float*)out, C, taps);
@@ -196,9 +267,11 @@ extern "C" int me_causal_conv(const void* x, int64_t x_stride, int dtype, const 
 }
 
 // ------------------------------------------------------------------ the recurrence
-// One wave per (request, head, 64 columns of P, NT rows of N, span of tokens). Lane p keeps column p of its NT state
-// rows in registers; the tokens' k and q slices, decays and input scales pass through LDS 16 tokens at a time and
-// are read from there by all lanes at once. Products and sums are float32 in the order of the tokens.
+// One wave per (request, one or two heads, 64 or 128 columns of P, NT rows of N, span of tokens). A lane keeps CL
+// columns of its NT state rows in registers (CL = 1, or 2: two blocks of 64 columns of one head, or the same 64
+// columns of two heads that share k and q); the tokens' k and q slices, decays and input scales pass through LDS 8
+// tokens at a time and are read from there by all lanes at once, while the next 8 tokens' values are already on
+// their way into registers. Products and sums are float32 in the order of the tokens.
 //
 // A launch is one of three passes (PASS):
 //   0  whole: a request's tokens from its state row, y written, the state row written back
@@ -219,20 +292,26 @@ struct RecArgs {
   float* y; int64_t y_slice_stride;                 // [slices of N, T, H * P] float32
   float* span_state; float* span_decay;             // scratch: [requests, spans, H, N, P], [requests, spans, H]
   int H, G, N, P, span, max_spans;
+  int silu;                                         // q, k and v pass silu on their way in
 };
 
-#define REC_TB 16
+#define REC_TB 8
 
-template <typename TX, int NT, int PASS>
+// HPB heads and PPB blocks of 64 columns per wave; CL = HPB * PPB columns per lane.
+template <typename TX, int NT, int PASS, int HPB, int PPB>
 __global__ void __launch_bounds__(64) recurrence_kernel(RecArgs a) {
-  __shared__ float sk[REC_TB][NT], sq[REC_TB][NT], sa[REC_TB], sb[REC_TB];
+  constexpr int CL = HPB * PPB;
+  constexpr int KR = REC_TB * NT / 64;               // k (and q) values a lane carries to LDS per batch of tokens
+  __shared__ float2 skq[REC_TB][NT];
+  __shared__ float sa[HPB][REC_TB], sb[HPB][REC_TB];
   const int lane = threadIdx.x;
-  const int bh = blockIdx.x, b = bh / a.H, h = bh - b * a.H;
-  const int g = h / (a.H / a.G);
-  const int p = blockIdx.y * 64 + lane;
-  const int n0 = blockIdx.z % ((a.N + NT - 1) / NT) * NT;
-  const int slice = blockIdx.z % ((a.N + NT - 1) / NT);
-  const int c = blockIdx.z / ((a.N + NT - 1) / NT);              // span index (0 in pass 0)
+  const int heads_blocks = a.H / HPB;
+  const int b = blockIdx.x / heads_blocks, h0 = (blockIdx.x - b * heads_blocks) * HPB;
+  const int g = h0 / (a.H / a.G);
+  const int slices = (a.N + NT - 1) / NT;
+  const int slice = blockIdx.z % slices;
+  const int c = blockIdx.z / slices;                  // span index (0 in pass 0)
+  const int n0 = slice * NT;
   const int64_t first = a.cu[b], end_all = a.cu[b + 1];
   int64_t t0 = first, t1 = end_all;
   if (PASS != 0) {
@@ -240,79 +319,157 @@ __global__ void __launch_bounds__(64) recurrence_kernel(RecArgs a) {
     t1 = t0 + a.span < end_all ? t0 + a.span : end_all;
   }
   if (t0 >= t1) return;
-  const bool on = p < a.P;
-  const int pc = on ? p : 0;
-  float S[NT];
-  float* row = a.state + (int64_t)a.slots[b] * a.state_stride + (int64_t)h * a.N * a.P;
-  float* span_row = PASS == 0 ? nullptr
-                              : a.span_state + (((int64_t)b * a.max_spans + c) * a.H + h) * (int64_t)a.N * a.P;
-  if (PASS == 1) {
+  int head[CL], p[CL];
+  bool on[CL];
 #pragma unroll
-    for (int i = 0; i < NT; ++i) S[i] = 0.f;
-  } else {
-    const float* from = PASS == 0 ? row : span_row;
-#pragma unroll
-    for (int i = 0; i < NT; ++i) S[i] = (on && n0 + i < a.N) ? from[(int64_t)(n0 + i) * a.P + pc] : 0.f;
+  for (int j = 0; j < CL; ++j) {
+    head[j] = h0 + (HPB == 2 ? j : 0);
+    p[j] = (blockIdx.y * PPB + (PPB == 2 ? j : 0)) * 64 + lane;
+    on[j] = p[j] < a.P;
+    if (!on[j]) p[j] = 0;
   }
   const TX* qp = (const TX*)a.q + (int64_t)g * a.N + n0;
   const TX* kp = (const TX*)a.k + (int64_t)g * a.N + n0;
-  const TX* vp = (const TX*)a.v + (int64_t)h * a.P + pc;
-  const float skip = a.skip ? a.skip[h] : 0.f;
-  float total_decay = 1.f;
-  for (int64_t tb = t0; tb < t1; tb += REC_TB) {
+  const bool silu = a.silu != 0;
+
+  // what a lane fetches for a batch of tokens
+  float kreg[KR], qreg[KR], vreg[CL][REC_TB], areg = 1.f, breg = 0.f;
+  // every load is unconditional, from an address clamped into the span and the slice; what lies outside becomes zero
+  // afterwards (a load behind a branch would make the wave wait for each one before it asks for the next)
+  const int n_last = a.N - 1 - n0;
+  auto fetch = [&](int64_t tb) {
     const int nt = (int)(t1 - tb < REC_TB ? t1 - tb : REC_TB);
-    __syncthreads();
-    for (int i = lane; i < REC_TB * NT; i += 64) {
-      const int tt = i / NT, nn = i - tt * NT;
-      const bool have = tt < nt && n0 + nn < a.N;
-      sk[tt][nn] = have ? to_f32<TX>(kp[(tb + tt) * a.k_stride + nn]) : 0.f;
-      if (PASS != 1) sq[tt][nn] = have ? to_f32<TX>(qp[(tb + tt) * a.q_stride + nn]) : 0.f;
-    }
-    if (lane < REC_TB) {
-      float da = 1.f, db = 0.f;
-      if (lane < nt) {
-        if (a.dt) {
-          const float z = to_f32<TX>(((const TX*)a.dt)[(tb + lane) * a.dt_stride + h]) + a.dt_bias[h];
-          const float step = z > 20.f ? z : log1pf(expf(z));
-          da = expf(-a.rate[h] * step);
-          db = step;
-        } else {
-          da = a.decay[h];
-          db = 1.f;
-        }
-      }
-      sa[lane] = da; sb[lane] = db;
-    }
-    float vv[REC_TB];
 #pragma unroll
-    for (int tt = 0; tt < REC_TB; ++tt) vv[tt] = (tt < nt && on) ? to_f32<TX>(vp[(tb + tt) * a.v_stride]) : 0.f;
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float da = sa[tt], bv = sb[tt] * vv[tt];
-      float acc = 0.f;
+    for (int r = 0; r < KR; ++r) {
+      const int i = lane + r * 64, tt = i / NT, nn = i - tt * NT;
+      const bool have = tt < nt && nn <= n_last;
+      const int64_t at = tb + (tt < nt ? tt : nt - 1);
+      const int col = nn <= n_last ? nn : n_last;
+      const float kk = to_f32<TX>(kp[at * a.k_stride + col]);
+      kreg[r] = have ? kk : 0.f;
+      if (PASS != 1) {
+        const float qq = to_f32<TX>(qp[at * a.q_stride + col]);
+        qreg[r] = have ? qq : 0.f;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < CL; ++j)
+#pragma unroll
+      for (int tt = 0; tt < REC_TB; ++tt) {
+        const float x = to_f32<TX>(((const TX*)a.v)[(tb + (tt < nt ? tt : nt - 1)) * a.v_stride + (int64_t)head[j] * a.P + p[j]]);
+        vreg[j][tt] = (tt < nt && on[j]) ? x : 0.f;
+      }
+    {
+      const int sub = lane < HPB * REC_TB ? lane : 0;
+      const int hh = h0 + sub / REC_TB, tt = sub % REC_TB;
+      const int64_t at = tb + (tt < nt ? tt : nt - 1);
+      if (a.dt) {
+        const float z = to_f32<TX>(((const TX*)a.dt)[at * a.dt_stride + hh]) + a.dt_bias[hh];
+        const float step = z > 20.f ? z : log1pf(expf(z));
+        areg = expf(-a.rate[hh] * step);
+        breg = step;
+      } else {
+        areg = a.decay[hh];
+        breg = 1.f;
+      }
+      if (tt >= nt) { areg = 1.f; breg = 0.f; }
+    }
+  };
+
+  fetch(t0);
+  float S[CL][NT];
+  float* row[CL];
+  float* span_row[CL];
+#pragma unroll
+  for (int j = 0; j < CL; ++j) {
+    row[j] = a.state + (int64_t)a.slots[b] * a.state_stride + (int64_t)head[j] * a.N * a.P;
+    span_row[j] = PASS == 0 ? nullptr : a.span_state + (((int64_t)b * a.max_spans + c) * a.H + head[j]) * (int64_t)a.N * a.P;
+    if (PASS == 1) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) S[j][i] = 0.f;
+    } else {
+      const float* from = PASS == 0 ? row[j] : span_row[j];
 #pragma unroll
       for (int i = 0; i < NT; ++i) {
-        S[i] = da * S[i] + sk[tt][i] * bv;
-        if (PASS != 1) acc += S[i] * sq[tt][i];
-      }
-      if (PASS == 1) total_decay *= da;
-      else if (on) {
-        if (slice == 0) acc += skip * vv[tt];
-        a.y[slice * a.y_slice_stride + (tb + tt) * ((int64_t)a.H * a.P) + (int64_t)h * a.P + p] = acc;
+        const float held = from[(int64_t)(n0 + (i <= n_last ? i : n_last)) * a.P + p[j]];
+        S[j][i] = (on[j] && i <= n_last) ? held : 0.f;
       }
     }
   }
-  if (PASS == 1) {
-    if (on)
+  float skip[CL];
+#pragma unroll
+  for (int j = 0; j < CL; ++j) skip[j] = a.skip ? a.skip[head[j]] : 0.f;
+  float total_decay[HPB];
+#pragma unroll
+  for (int j = 0; j < HPB; ++j) total_decay[j] = 1.f;
+
+  for (int64_t tb = t0; tb < t1; tb += REC_TB) {
+    const int nt = (int)(t1 - tb < REC_TB ? t1 - tb : REC_TB);
+    __syncthreads();                                  // the batch before has been read
+    float vv[CL][REC_TB];
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+      const int i = lane + r * 64, tt = i / NT, nn = i - tt * NT;
+      float kk = kreg[r], qq = PASS != 1 ? qreg[r] : 0.f;
+      if (silu) { kk = silu_f(kk); qq = silu_f(qq); }
+      skq[tt][nn] = make_float2(kk, qq);
+    }
+    if (lane < HPB * REC_TB) { sa[lane / REC_TB][lane % REC_TB] = areg; sb[lane / REC_TB][lane % REC_TB] = breg; }
+#pragma unroll
+    for (int j = 0; j < CL; ++j)
+#pragma unroll
+      for (int tt = 0; tt < REC_TB; ++tt) vv[j][tt] = silu ? silu_f(vreg[j][tt]) : vreg[j][tt];
+    if (tb + REC_TB < t1) fetch(tb + REC_TB);         // the next batch travels while this one is computed
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < REC_TB; ++tt) {
+      if (tt >= nt) break;
+      float da[CL], bv[CL], acc[CL];
+#pragma unroll
+      for (int j = 0; j < CL; ++j) {
+        const int hj = HPB == 2 ? j : 0;
+        da[j] = sa[hj][tt];
+        bv[j] = sb[hj][tt] * vv[j][tt];
+        acc[j] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const float2 kq = skq[tt][i];
+#pragma unroll
+        for (int j = 0; j < CL; ++j) {
+          S[j][i] = da[j] * S[j][i] + kq.x * bv[j];
+          if (PASS != 1) acc[j] += S[j][i] * kq.y;
+        }
+      }
+      if (PASS == 1) {
+#pragma unroll
+        for (int j = 0; j < HPB; ++j) total_decay[j] *= sa[j][tt];
+      } else {
+#pragma unroll
+        for (int j = 0; j < CL; ++j)
+          if (on[j]) {
+            if (slice == 0) acc[j] += skip[j] * vv[j][tt];
+            a.y[slice * a.y_slice_stride + (tb + tt) * ((int64_t)a.H * a.P) + (int64_t)head[j] * a.P + p[j]] = acc[j];
+          }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < CL; ++j) {
+    if (PASS == 1) {
+      if (on[j])
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+          if (n0 + i < a.N) span_row[j][(int64_t)(n0 + i) * a.P + p[j]] = S[j][i];
+    } else if (on[j] && t1 == end_all) {
 #pragma unroll
       for (int i = 0; i < NT; ++i)
-        if (n0 + i < a.N) span_row[(int64_t)(n0 + i) * a.P + p] = S[i];
-    if (lane == 0 && blockIdx.y == 0 && slice == 0) a.span_decay[((int64_t)b * a.max_spans + c) * a.H + h] = total_decay;
-  } else if (on && t1 == end_all) {
-#pragma unroll
-    for (int i = 0; i < NT; ++i)
-      if (n0 + i < a.N) row[(int64_t)(n0 + i) * a.P + p] = S[i];
+        if (n0 + i < a.N) row[j][(int64_t)(n0 + i) * a.P + p[j]] = S[j][i];
+    }
   }
+  if (PASS == 1 && lane == 0 && blockIdx.y == 0 && slice == 0)
+#pragma unroll
+    for (int j = 0; j < HPB; ++j) a.span_decay[((int64_t)b * a.max_spans + c) * a.H + h0 + j] = total_decay[j];
 }
 
 // in[0] = the request's state row; in[c + 1] = decay[c] * in[c] + end[c]. scratch[c] holds end[c] on entry and in[c] on
@@ -335,59 +492,73 @@ __global__ void recurrence_carry_kernel(RecArgs a) {
   }
 }
 
-template <typename TX, int NT>
+template <typename TX, int NT, int HPB, int PPB>
 static int launch_recurrence(RecArgs& a, int num_seqs, int spans, hipStream_t stream) {
   const int slices = (a.N + NT - 1) / NT;
   const dim3 block(64);
+  const unsigned pblocks = (a.P + 64 * PPB - 1) / (64 * PPB);
   if (spans <= 1) {
-    recurrence_kernel<TX, NT, 0><<<dim3(num_seqs * a.H, (a.P + 63) / 64, slices), block, 0, stream>>>(a);
+    recurrence_kernel<TX, NT, 0, HPB, PPB><<<dim3(num_seqs * (a.H / HPB), pblocks, slices), block, 0, stream>>>(a);
     ME_LAUNCH_CHECK();
     return 0;
   }
-  const dim3 grid(num_seqs * a.H, (a.P + 63) / 64, slices * spans);
-  recurrence_kernel<TX, NT, 1><<<grid, block, 0, stream>>>(a);
+  const dim3 grid(num_seqs * (a.H / HPB), pblocks, slices * spans);
+  recurrence_kernel<TX, NT, 1, HPB, PPB><<<grid, block, 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   const int64_t per_req = (int64_t)a.H * a.N * a.P;
   recurrence_carry_kernel<<<dim3((unsigned)((per_req + 255) / 256), num_seqs), dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
-  recurrence_kernel<TX, NT, 2><<<grid, block, 0, stream>>>(a);
+  recurrence_kernel<TX, NT, 2, HPB, PPB><<<grid, block, 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   return 0;
 }
 
 // spans <= 1: every request's tokens in one pass. Otherwise the tokens are cut into spans of `span` tokens that run
 // side by side (at most `spans` per request), and scratch holds spans * H * N * P + spans * H floats per request.
+// columns: 1, or 2: a lane keeps two columns of the state (two blocks of 64 columns of one head where P > 64, else
+// the same columns of two neighbouring heads of one group, which needs an even number of heads per group).
 extern "C" int me_linear_recurrence(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                     int64_t v_stride, int dtype, const void* dt, int64_t dt_stride, const float* decay,
                                     const float* dt_bias, const float* rate, const float* skip, float* state,
                                     int64_t state_stride, const int32_t* slots, const int32_t* cu, float* y,
                                     int64_t y_slice_stride, int num_seqs, int H, int G, int N, int P, int rows_per_wave,
-                                    int span, int spans, float* scratch, hipStream_t stream) {
+                                    int columns, int silu, int span, int spans, float* scratch, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   ME_CHECK(H >= 1 && G >= 1 && H % G == 0 && N >= 1 && P >= 1, "recurrence: bad sizes H=%d G=%d N=%d P=%d", H, G, N, P);
   ME_CHECK((dt != nullptr) != (decay != nullptr), "recurrence: give fixed decays or step sizes, not both");
   ME_CHECK(dt == nullptr || (dt_bias && rate), "recurrence: step sizes need their bias and rates");
   ME_CHECK((int64_t)num_seqs * H <= 2147483647ll, "recurrence: too many (request, head) pairs");
   ME_CHECK(spans <= 1 || (span >= 1 && scratch != nullptr), "recurrence: spans need a length and scratch");
+  const bool two_heads = columns == 2 && P <= 64;
+  ME_CHECK(columns == 1 || columns == 2, "recurrence: 1 or 2 columns per lane");
+  ME_CHECK(!two_heads || (H / G) % 2 == 0, "recurrence: two heads per wave need an even number of heads per group");
   RecArgs a;
   a.q = q; a.k = k; a.v = v; a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
   a.dt = dt; a.dt_stride = dt_stride; a.decay = decay; a.dt_bias = dt_bias; a.rate = rate; a.skip = skip;
   a.state = state; a.state_stride = state_stride; a.slots = slots; a.cu = cu; a.y = y; a.y_slice_stride = y_slice_stride;
   a.H = H; a.G = G; a.N = N; a.P = P; a.span = span > 0 ? span : 1; a.max_spans = spans > 1 ? spans : 1;
+  a.silu = silu;
   a.span_state = scratch;
   a.span_decay = scratch ? scratch + (int64_t)num_seqs * a.max_spans * H * N * P : nullptr;
   const int slices = (N + rows_per_wave - 1) / rows_per_wave;
   ME_CHECK((int64_t)slices * a.max_spans <= 65535, "recurrence: too many slices and spans for one launch");
+#define REC_NT(TX, NT)                                                                               \
+  do {                                                                                               \
+    if (columns == 1) return launch_recurrence<TX, NT, 1, 1>(a, num_seqs, spans, stream);            \
+    if (two_heads) return launch_recurrence<TX, NT, 2, 1>(a, num_seqs, spans, stream);               \
+    return launch_recurrence<TX, NT, 1, 2>(a, num_seqs, spans, stream);                              \
+  } while (0)
 #define REC(TX)                                                                              \
   switch (rows_per_wave) {                                                                   \
-    case 16: return launch_recurrence<TX, 16>(a, num_seqs, spans, stream);                   \
-    case 32: return launch_recurrence<TX, 32>(a, num_seqs, spans, stream);                   \
-    case 48: return launch_recurrence<TX, 48>(a, num_seqs, spans, stream);                   \
-    case 64: return launch_recurrence<TX, 64>(a, num_seqs, spans, stream);                   \
+    case 16: REC_NT(TX, 16);                                                                 \
+    case 32: REC_NT(TX, 32);                                                                 \
+    case 48: REC_NT(TX, 48);                                                                 \
+    case 64: REC_NT(TX, 64);                                                                 \
     default: ME_CHECK(false, "recurrence: %d state rows per wave is not one of 16, 32, 48, 64", rows_per_wave); \
   }
   if (dtype == ME_F32) { REC(float) } else { REC(bf16_t) }
 #undef REC
+#undef REC_NT
   return 0;
 }
 

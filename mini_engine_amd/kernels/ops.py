@@ -75,7 +75,7 @@ _CORE_PROTOS = {
     "me_activation": [P, L, P, I, I, L, I, P],
     "me_head_gate": [P, P, L, I, L, I, I, P],
     "me_causal_conv": [P, L, I, P, P, P, L, P, P, P, P, L, I, I, I, P],
-    "me_linear_recurrence": [P, L, P, L, P, L, I, P, L, P, P, P, P, P, L, P, P, P, L, I, I, I, I, I, I, I, I, P, P],
+    "me_linear_recurrence": [P, L, P, L, P, L, I, P, L, P, P, P, P, P, L, P, P, P, L, I, I, I, I, I, I, I, I, I, I, P, P],
     "me_gated_rms_norm": [P, I, L, P, L, I, P, P, L, I, I, I, F, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
@@ -633,13 +633,13 @@ class HipBackend:
         return out
 
     def linear_recurrence(self, q, k, v, state, state_slots, cu_seqlens, q_lens, H: int, G: int, N: int, P: int,
-                          decay=None, dt=None, dt_bias=None, rate=None, skip=None) -> torch.Tensor:
+                          decay=None, dt=None, dt_bias=None, rate=None, skip=None, silu: bool = False) -> torch.Tensor:
         """Per request and head, over the request's tokens of this step in order, from its state row:
             S_t = a_t S_(t-1) + b_t k_t v_t^T,   y_t = S_t^T q_t (+ skip_h v_t),      S [N, P] float32.
         q, k: row views [T, G * N] (heads share them by groups of H / G), v: [T, H * P]; state: float32 view
         [slots, H * N * P], rows `state_slots`, left at the state behind the last token. a, b: `decay` (float32 [H])
         and 1; or exp(-rate_h dt), dt with dt = softplus(dt[t, h] + dt_bias_h) (`dt` a row view [T, H], the others
-        float32 [H]). `q_lens`: the requests' token counts on the host: long ones are cut into spans that run side
+        float32 [H]). `silu`: q, k and v pass silu on their way in. `q_lens`: the requests' token counts on the host: long ones are cut into spans that run side
         by side (`recurrence_spans`). Returns float32 [T, H * P], or partial sums [S, T, H * P] over slices of N
         for a consumer that adds them."""
         T, B = v.shape[0], state_slots.numel()
@@ -657,13 +657,14 @@ class HipBackend:
         _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B, "recurrence: metadata")
         per_wave = recurrence_rows_per_wave(N)
         slices = -(-N // per_wave)
-        span, spans = recurrence_spans(q_lens, H * -(-P // 64) * slices)
+        columns = recurrence_columns(q_lens, H, G, P, slices)
+        span, spans = recurrence_spans(q_lens, H * -(-P // 64) * slices // columns)
         scratch = _scratch(B * spans * (H * N * P + H), v.device, "recurrence") if spans > 1 else None
         y = torch.empty((slices, T, H * P) if slices > 1 else (T, H * P), dtype=torch.float32, device=v.device)
         core().call("me_linear_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
                     _code(dtype), _ptr(dt), 0 if dt is None else dt.stride(0), _ptr(decay), _ptr(dt_bias), _ptr(rate), _ptr(skip),
                     state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), y.data_ptr(), T * H * P,
-                    B, H, G, N, P, per_wave, span, spans, _ptr(scratch), _stream())
+                    B, H, G, N, P, per_wave, columns, int(silu), span, spans, _ptr(scratch), _stream())
         return y
 
     def gated_rms_norm(self, y, gate, weight, eps: float, groups: int, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
@@ -1100,6 +1101,20 @@ def recurrence_rows_per_wave(N: int) -> int:
     return min((64, 48, 32), key=lambda r: (-(-N // r) * r - N, -r))
 
 
+def recurrence_columns(q_lens: list, H: int, G: int, P: int, slices: int) -> int:
+    """State columns a lane of the recurrence kernel keeps: 1. The kernel also has a form with 2 (two blocks of 64
+    columns of one head where P exceeds 64, else the same columns of two neighbouring heads of a group, which needs
+    an even number of heads per group): it halves the reads of k and q from LDS per product, but its 256 registers
+    leave one wave to a SIMD, and it measured slower at every size tried (a prompt of 2,048 tokens at 16 heads of
+    128 x 128: 283 against 222 us; 64 requests decoding: 98 against 54 us). ME_RECURRENCE_COLUMNS=2 forces it, for
+    timing one against the other."""
+    if RECURRENCE_COLUMNS == 2 and not (P <= 64 and (H // G) % 2):
+        return 2
+    return 1
+
+
+import os as _os
+RECURRENCE_COLUMNS = int(_os.environ.get("ME_RECURRENCE_COLUMNS", "0"))     # 1 or 2 force the columns per lane (for timing one against the other)
 RECURRENCE_MIN_SPAN = 64
 RECURRENCE_WAVES = 2048        # waves that keep the 256 compute units busy: 8 a unit
 

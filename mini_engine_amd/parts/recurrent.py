@@ -48,9 +48,9 @@ class LinearAttention(Mixer):
     def forward(self, x, step, cache, state):
         H, N, P = self.num_heads, self.key_dim, self.value_dim
         rows = self.qkvg.forward(x)                                   # [T, q | k | v | g]
-        qkv = ops.activation(rows[:, : 2 * self.qk + self.inner], "silu")
-        y = ops.linear_recurrence(qkv[:, : self.qk], qkv[:, self.qk: 2 * self.qk], qkv[:, 2 * self.qk:], state,
-                                  step.state_slots, step.cu_seqlens, step.q_lens, H, H, N, P, decay=self.decay)
+        # silu of q, k and v happens where the recurrence reads them (float32, unrounded)
+        y = ops.linear_recurrence(rows[:, : self.qk], rows[:, self.qk: 2 * self.qk], rows[:, 2 * self.qk: 2 * self.qk + self.inner],
+                                  state, step.state_slots, step.cu_seqlens, step.q_lens, H, H, N, P, decay=self.decay, silu=True)
         o = ops.gated_rms_norm(y, rows[:, 2 * self.qk + self.inner:], self.norm_weight, self.norm_eps, 1, "sigmoid_behind",
                                rows.dtype)
         return self.o.forward(o, allow_partials=True)

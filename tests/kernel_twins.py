@@ -210,7 +210,7 @@ def softplus(x):
 
 
 def linear_recurrence(q, k, v, state, state_slots, cu_seqlens, q_lens, H, G, N, P, decay=None, dt=None, dt_bias=None,
-                      rate=None, skip=None):
+                      rate=None, skip=None, silu=False):
     """S_t = a S_(t-1) + b k_t v_t^T, y_t = S_t^T q_t (+ skip v_t), float32, token by token. q, k [T, G * N], v [T, H * P];
     state [slots, H * N * P]. a, b: decay[h], 1; or exp(-rate[h] dt), dt with dt = softplus(dt[t, h] + dt_bias[h])."""
     T = v.shape[0]
@@ -221,6 +221,8 @@ def linear_recurrence(q, k, v, state, state_slots, cu_seqlens, q_lens, H, G, N, 
         S = state[slots[b]].view(H, N, P).clone()
         for t in range(cu[b], cu[b + 1]):
             kt, qt, vt = k[t].float().view(G, N), q[t].float().view(G, N), v[t].float().view(H, P)
+            if silu:
+                kt, qt, vt = (z * torch.sigmoid(z) for z in (kt, qt, vt))
             if decay is not None:
                 a, bb = decay.float(), torch.ones(H)
             else:
