@@ -492,6 +492,68 @@ __global__ void recurrence_carry_kernel(RecArgs a) {
   }
 }
 
+// A step of single tokens (token b is request b's): the state streams through once. One workgroup of four waves per
+// (request, head, 64 columns); each wave takes a quarter of the N rows, eight rows' loads in flight at a time, and
+// the four partial outputs meet in LDS. Nothing of the state stays in registers, so many waves fit a SIMD, which is
+// what a kernel that only waits for memory needs.
+template <typename TX>
+__global__ void __launch_bounds__(256) recurrence_step_kernel(RecArgs a) {
+  extern __shared__ float kq[];                       // k[N], q[N], then 4 x 64 partial outputs
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.x / a.H, h = blockIdx.x - b * a.H;
+  const int g = h / (a.H / a.G);
+  const int p = blockIdx.y * 64 + lane;
+  const bool on = p < a.P;
+  const int pc = on ? p : 0;
+  float* sk = kq;
+  float* sq = kq + a.N;
+  float* part = kq + 2 * a.N;
+  const bool silu = a.silu != 0;
+  for (int i = threadIdx.x; i < a.N; i += 256) {
+    float kk = to_f32<TX>(((const TX*)a.k)[(int64_t)b * a.k_stride + (int64_t)g * a.N + i]);
+    float qq = to_f32<TX>(((const TX*)a.q)[(int64_t)b * a.q_stride + (int64_t)g * a.N + i]);
+    if (silu) { kk = silu_f(kk); qq = silu_f(qq); }
+    sk[i] = kk; sq[i] = qq;
+  }
+  float vv = to_f32<TX>(((const TX*)a.v)[(int64_t)b * a.v_stride + (int64_t)h * a.P + pc]);
+  if (silu) vv = silu_f(vv);
+  float da, db;
+  if (a.dt) {
+    const float z = to_f32<TX>(((const TX*)a.dt)[(int64_t)b * a.dt_stride + h]) + a.dt_bias[h];
+    const float step = z > 20.f ? z : log1pf(expf(z));
+    da = expf(-a.rate[h] * step);
+    db = step;
+  } else {
+    da = a.decay[h];
+    db = 1.f;
+  }
+  const float bv = db * vv;
+  float* row = a.state + (int64_t)a.slots[b] * a.state_stride + (int64_t)h * a.N * a.P + pc;
+  const int per = (a.N + 3) / 4;
+  const int r0 = wave * per, r1 = r0 + per < a.N ? r0 + per : a.N;
+  __syncthreads();
+  float acc = 0.f;
+  for (int r = r0; r < r1; r += 8) {
+    float held[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) held[i] = row[(int64_t)(r + i < r1 ? r + i : r1 - 1) * a.P];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (r + i < r1) {
+        const float next = da * held[i] + sk[r + i] * bv;
+        acc += next * sq[r + i];
+        if (on) row[(int64_t)(r + i) * a.P] = next;
+      }
+  }
+  part[wave * 64 + lane] = acc;
+  __syncthreads();
+  if (wave == 0 && on) {
+    float y = part[lane] + part[64 + lane] + part[128 + lane] + part[192 + lane];
+    if (a.skip) y += a.skip[h] * vv;
+    a.y[(int64_t)b * a.H * a.P + (int64_t)h * a.P + p] = y;
+  }
+}
+
 template <typename TX, int NT, int HPB, int PPB>
 static int launch_recurrence(RecArgs& a, int num_seqs, int spans, hipStream_t stream) {
   const int slices = (a.N + NT - 1) / NT;
@@ -540,6 +602,15 @@ extern "C" int me_linear_recurrence(const void* q, int64_t q_stride, const void*
   a.silu = silu;
   a.span_state = scratch;
   a.span_decay = scratch ? scratch + (int64_t)num_seqs * a.max_spans * H * N * P : nullptr;
+  if (rows_per_wave == 0) {                // a step of single tokens: one pass over the state, one output
+    ME_CHECK((int64_t)(2 * N + 256) * 4 <= 64 * 1024 && (P + 63) / 64 <= 65535, "recurrence: a state of %d rows does not fit the step kernel", N);
+    const dim3 grid(num_seqs * H, (P + 63) / 64);
+    const size_t lds = (size_t)(2 * N + 256) * sizeof(float);
+    if (dtype == ME_F32) recurrence_step_kernel<float><<<grid, dim3(256), lds, stream>>>(a);
+    else recurrence_step_kernel<bf16_t><<<grid, dim3(256), lds, stream>>>(a);
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   const int slices = (N + rows_per_wave - 1) / rows_per_wave;
   ME_CHECK((int64_t)slices * a.max_spans <= 65535, "recurrence: too many slices and spans for one launch");
 #define REC_NT(TX, NT)                                                                               \

@@ -655,6 +655,14 @@ class HipBackend:
             _check(dt.shape == (T, H) and dt.stride(1) == 1 and dt.dtype == dtype and dt_bias is not None and rate is not None,
                    "recurrence: step sizes [T, H] with bias and rates")
         _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B, "recurrence: metadata")
+        if T == B and N <= RECURRENCE_STEP_MAX_ROWS:
+            # every request brings one token: the state streams through once, one output row per token
+            y = torch.empty((T, H * P), dtype=torch.float32, device=v.device)
+            core().call("me_linear_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                        _code(dtype), _ptr(dt), 0 if dt is None else dt.stride(0), _ptr(decay), _ptr(dt_bias), _ptr(rate), _ptr(skip),
+                        state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), y.data_ptr(), T * H * P,
+                        B, H, G, N, P, 0, 1, int(silu), 0, 1, None, _stream())
+            return y
         per_wave = recurrence_rows_per_wave(N)
         slices = -(-N // per_wave)
         columns = recurrence_columns(q_lens, H, G, P, slices)
@@ -1114,6 +1122,7 @@ def recurrence_columns(q_lens: list, H: int, G: int, P: int, slices: int) -> int
 
 
 import os as _os
+RECURRENCE_STEP_MAX_ROWS = 4096     # state rows up to which the single-token kernel's k and q fit its LDS
 RECURRENCE_COLUMNS = int(_os.environ.get("ME_RECURRENCE_COLUMNS", "0"))     # 1 or 2 force the columns per lane (for timing one against the other)
 RECURRENCE_MIN_SPAN = 64
 RECURRENCE_WAVES = 2048        # waves that keep the 256 compute units busy: 8 a unit

@@ -111,12 +111,17 @@ def test_causal_conv_continues_from_its_state(dtype, taps, C):
     assert torch.equal(torch.cat((first, rest)), got[T - 37:]) and torch.equal(st2[2], st_h[2])
 
 
+@pytest.mark.parametrize("columns", [1, 2])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,N,P,selective", [(4, 2, 20, 12, True), (3, 3, 10, 20, False), (2, 1, 70, 80, True),
                                                (2, 2, 130, 8, False), (5, 1, 48, 48, True), (8, 8, 64, 64, False)])
-def test_linear_recurrence(dtype, H, G, N, P, selective):
+def test_linear_recurrence(monkeypatch, dtype, H, G, N, P, selective, columns):
     """Requests of unequal lengths from states of their own, against the token-by-token twin; 300 tokens are cut into
-    spans that run side by side (the launch rule says so), which must give what one pass gives."""
+    spans that run side by side (the launch rule says so), which must give what one pass gives. Both forms of the
+    kernel: one state column per lane, and two (blocks of one head, or two heads of a group)."""
+    monkeypatch.setattr(ops, "RECURRENCE_COLUMNS", columns)
+    assert ops.recurrence_columns([300], H, G, P, 1) == (1 if columns == 1 or (P <= 64 and (H // G) % 2) else 2)
+    silu = not selective and H == 3
     torch.manual_seed(H * N + P)
     q_lens = [1, 300, 2, 17]
     cu, seq, slots = _steps_meta(q_lens, [2, 0, 4, 1])
@@ -129,13 +134,13 @@ def test_linear_recurrence(dtype, H, G, N, P, selective):
         kw = dict(dt=rows[:, 1 + 2 * G * N + H * P:1 + 2 * G * N + H * P + H], dt_bias=torch.randn(H, device=DEV) - 2,
                   rate=torch.rand(H, device=DEV) * 4 + 0.2, skip=torch.randn(H, device=DEV))
     else:
-        kw = dict(decay=torch.tensor([0.5, 0.9, 0.99, 0.999, 0.8, 0.95, 0.7, 0.9999][:H], device=DEV))
+        kw = dict(decay=torch.tensor([0.5, 0.9, 0.99, 0.999, 0.8, 0.95, 0.7, 0.9999][:H], device=DEV), silu=silu)
     full = torch.randn(6, 3 + H * N * P, device=DEV)
     st_h, st_c = full.clone(), full.cpu().clone()
     assert ops.recurrence_spans(q_lens, 1)[1] > 1
     y = hip().linear_recurrence(q, k, v, st_h[:, 3:], slots, cu, q_lens, H, G, N, P, **kw)
     y = y.sum(0) if y.dim() == 3 else y
-    cpu = {n: t.cpu() for n, t in kw.items()}
+    cpu = {n: (t.cpu() if torch.is_tensor(t) else t) for n, t in kw.items()}
     want = twin.linear_recurrence(q.cpu(), k.cpu(), v.cpu(), st_c[:, 3:], slots.cpu(), cu.cpu(), q_lens, H, G, N, P, **cpu)
     tol = 2e-5 if dtype == torch.float32 else 2e-5        # the inputs are exact in both; only the sums' order differs
     close(y, want, tol)
@@ -148,6 +153,17 @@ def test_linear_recurrence(dtype, H, G, N, P, selective):
     one = torch.cat([o.sum(0) if o.dim() == 3 else o for o in one])
     close(one, want[T - 17:], tol)
     close(st1[1], st_c[1], tol)
+    # five requests with one token each (the kernel of pure decode steps), slots in an order of their own
+    st5, st5c = full.clone(), full.cpu().clone()
+    cu5, _, sl5 = _steps_meta([1] * 5, [4, 0, 2, 5, 1])
+    kw5 = {n: (a[:5] if n == "dt" else a) for n, a in kw.items()}
+    got5 = hip().linear_recurrence(q[:5], k[:5], v[:5], st5[:, 3:], sl5, cu5, [1] * 5, H, G, N, P, **kw5)
+    assert got5.dim() == 2
+    want5 = twin.linear_recurrence(q[:5].cpu(), k[:5].cpu(), v[:5].cpu(), st5c[:, 3:], sl5.cpu(), cu5.cpu(), [1] * 5, H, G, N, P,
+                                   **{n: (t.cpu() if torch.is_tensor(t) else t) for n, t in kw5.items()})
+    close(got5, want5, tol)
+    close(st5, st5c, tol)
+    assert torch.equal(st5[3], full[3]) and torch.equal(st5[:, :3], full[:, :3])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
