@@ -317,7 +317,11 @@ def resolve_model(args, size: str, layers, tmp: str) -> tuple:
         cfg = load_model_config(size)
         label = os.path.basename(os.path.normpath(size))
         full = getattr(cfg, "num_hidden_layers", None)
-        if checkpoint_files(size):
+        try:
+            stored = checkpoint_files(size)
+        except ValueError:                   # a folder with config.json only
+            stored = []
+        if stored:
             return cfg, full, label, size, None, "the folder's checkpoint"
         return cfg, full, label, size, args.seed, "drawn on the device"
     design = size.startswith("sigosun:")

@@ -39,52 +39,80 @@ __global__ void add_rms_norm_kernel(const TX* __restrict__ y, int parts, int64_t
   }
 }
 
-// The same with every operand of a row asked for at once and kept in registers (rows of up to BD * 8 elements): one
-// trip to memory before the workgroup's sum and none behind it, which is what a step of a few rows waits for.
+// The same for rows of up to 4,096 elements in whole groups of 4: a thread owns one group, asks for every operand of it
+// at once (each partial sum, the stream, the weight) and keeps it in registers: one trip to memory before the
+// workgroup's sum and none behind it, which is what a step of a few rows waits for.
+template <typename T> struct Group4;
+template <> struct Group4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Group4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(t[i]);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    bf16x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = static_cast<bf16_t>(v[i]);
+    *reinterpret_cast<bf16x4*>(p) = t;
+  }
+};
+
 template <typename TX, typename TY>
 __global__ void add_rms_norm_regs_kernel(const TX* __restrict__ y, int parts, int64_t part_stride, const float* __restrict__ w,
                                          const float* __restrict__ stream_in, float* __restrict__ stream_out,
                                          TY* __restrict__ rounded, int n, float eps) {
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
-  const TX* yr = y + t * n;
-  float yv[8], sv[8], wv[8];
-  float ss = 0.f;
+  const int i = threadIdx.x * 4;
+  const bool on = i < n;
+  float part[RC_MAX_PARTIALS][4], sv[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f}, yv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (on) {
 #pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    const int i = threadIdx.x + k * blockDim.x;
-    yv[k] = 0.f; sv[k] = 0.f; wv[k] = 0.f;
-    if (i < n) {
-      for (int p = 0; p < parts; ++p) yv[k] += to_f32<TX>(yr[p * part_stride + i]);
-      sv[k] = stream_in[t * n + i];
-      wv[k] = w[i];
-    }
-    ss += yv[k] * yv[k];
+    for (int p = 0; p < RC_MAX_PARTIALS; ++p)
+      if (p < parts) Group4<TX>::load(y + p * part_stride + t * n + i, part[p]);
+    Group4<float>::load(stream_in + t * n + i, sv);
+    Group4<float>::load(w + i, wv);
+#pragma unroll
+    for (int p = 0; p < RC_MAX_PARTIALS; ++p)
+      if (p < parts) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[e] += part[p][e];
+      }
   }
+  float ss = yv[0] * yv[0] + yv[1] * yv[1] + yv[2] * yv[2] + yv[3] * yv[3];
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  if (on) {
+    float r[4];
 #pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    const int i = threadIdx.x + k * blockDim.x;
-    if (i < n) {
-      const float r = sv[k] + yv[k] * inv * wv[k];
-      stream_out[t * n + i] = r;
-      if (rounded) rounded[t * n + i] = from_f32<TY>(r);
-    }
+    for (int e = 0; e < 4; ++e) r[e] = sv[e] + yv[e] * inv * wv[e];
+    Group4<float>::store(stream_out + t * n + i, r);
+    if (rounded) Group4<TY>::store(rounded + t * n + i, r);
   }
 }
 
 template <typename TX, typename TY>
 static void launch_add_rms_norm(const TX* y, int parts, int64_t part_stride, const float* w, const float* stream_in,
                                 float* stream_out, TY* rounded, int64_t T, int n, float eps, hipStream_t stream) {
-  if (n <= 8192) {
-    const int threads = n <= 512 ? 64 : (n <= 2048 ? 256 : 1024);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(stream_in) |
+                         reinterpret_cast<uintptr_t>(stream_out) | reinterpret_cast<uintptr_t>(rounded)) % 16) == 0;
+  if (n <= 4096 && n % 4 == 0 && aligned && (parts == 1 || part_stride % 4 == 0)) {
+    const int threads = ((n / 4) + 63) / 64 * 64;
     add_rms_norm_regs_kernel<TX, TY><<<dim3((unsigned)T), dim3(threads), 0, stream>>>(y, parts, part_stride, w, stream_in,
                                                                                      stream_out, rounded, n, eps);
     return;
   }
-  add_rms_norm_kernel<TX, TY><<<dim3((unsigned)T), dim3(256), (size_t)n * sizeof(float), stream>>>(y, parts, part_stride, w, stream_in,
-                                                                                                 stream_out, rounded, n, eps);
+  add_rms_norm_kernel<TX, TY><<<dim3((unsigned)T), dim3(n >= 1024 ? 256 : (n > 256 ? 128 : 64)), (size_t)n * sizeof(float), stream>>>(
+      y, parts, part_stride, w, stream_in, stream_out, rounded, n, eps);
 }
 
 extern "C" int me_add_rms_norm(const void* y, int y_dtype, int parts, int64_t part_stride, const float* w,
