@@ -679,6 +679,8 @@ class HipBackend:
         """`kind` "silu_before": u = y * silu(gate), out = u / rms(u) * weight with the root mean square taken over
         each of `groups` equal parts of a row; "sigmoid_behind": out = y / rms(y) * weight * sigmoid(gate). y float32
         [T, n] or slices [S, T, n] that are added first; gate a row view [T, n] of out_dtype. Returns [T, n]."""
+        if y.dim() == 3 and y.shape[0] > 64:          # more slices than the kernel adds (a state of thousands of rows)
+            y = y.sum(0)
         parts = y.shape[0] if y.dim() == 3 else 1
         T, n = y.shape[-2], y.shape[-1]
         _check(y.dtype == torch.float32 and y.is_contiguous() and kind in GATED_NORMS, "gated_rms_norm: float32 rows, a known kind")
@@ -1102,11 +1104,13 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
 
 
 def recurrence_rows_per_wave(N: int) -> int:
-    """State rows a wave of the recurrence kernel keeps in registers per lane (16, 32, 48 or 64): all of N up to 64,
-    beyond that the size that wastes the fewest rows over its slices (ties to the larger)."""
-    if N <= 64:
+    """State rows a wave of the recurrence kernel keeps in registers per lane (16, 32, 48 or 64): all of N up to 48,
+    beyond that slices of 32 (or of 48 where they waste fewer rows): four waves to a SIMD then share its LDS reads
+    and hide each other's waits, where slices of 64 leave two (a prompt of 2,048 tokens at 16 heads of 128 x 128: 185
+    against 221 us; 8,192 tokens: 644 against 698)."""
+    if N <= 48:
         return -(-N // 16) * 16
-    return min((64, 48, 32), key=lambda r: (-(-N // r) * r - N, -r))
+    return min((32, 48), key=lambda r: (-(-N // r) * r - N, r))
 
 
 def recurrence_columns(q_lens: list, H: int, G: int, P: int, slices: int) -> int:
@@ -1125,7 +1129,7 @@ import os as _os
 RECURRENCE_STEP_MAX_ROWS = 4096     # state rows up to which the single-token kernel's k and q fit its LDS
 RECURRENCE_COLUMNS = int(_os.environ.get("ME_RECURRENCE_COLUMNS", "0"))     # 1 or 2 force the columns per lane (for timing one against the other)
 RECURRENCE_MIN_SPAN = 64
-RECURRENCE_WAVES = 2048        # waves that keep the 256 compute units busy: 8 a unit
+RECURRENCE_WAVES = 4096        # waves that keep the 256 compute units busy: 16 a unit, 4 a SIMD
 
 
 def recurrence_spans(q_lens: list, waves_per_request: int) -> tuple:
@@ -1134,8 +1138,9 @@ def recurrence_spans(q_lens: list, waves_per_request: int) -> tuple:
     A request's tokens are a chain, and one pass gives the GPU only requests x heads x slices waves. A long prompt is
     therefore cut into spans that run side by side: each span first from zero, then a walk over the spans' end states
     carries the state on, then each span again from the state before it, which costs the work twice and pays as soon
-    as the spans are many. Spans of RECURRENCE_MIN_SPAN tokens or more, as many as bring the launch to
-    RECURRENCE_WAVES waves, for steps whose longest request has two spans or more."""
+    as the spans are many. Spans of RECURRENCE_MIN_SPAN tokens or more (shorter ones spend their time on reading and
+    writing states), as many as bring the launch to RECURRENCE_WAVES waves, for steps whose longest request has two
+    spans or more."""
     longest = max(q_lens, default=0)
     if longest < 2 * RECURRENCE_MIN_SPAN:
         return 0, 1

@@ -65,8 +65,16 @@ CONFIGS = {
     "far": _model(80, 32, 1e-5, [_att(3, 1, 32, 16, 0.2, 32, 250000.0, 300, ff=40), _lin(1, 16, 16, [0.999]),
                                  _att(3, 1, 32, 16, 0.2, 32, 250000.0, 64, kv_from=0, ff=40)]),
 }
-SEEDS = {"mix": 11, "att": 12, "ssm": 13, "lin": 14, "far": 15}
-PAGE = {"mix": 8, "att": 16, "ssm": 16, "lin": 8, "far": 16}
+# the layer sizes of a real model (heads of 128, a state of 128 x 64, four taps), few layers: the kernel forms that
+# the small widths above never reach
+CONFIGS["real"] = _model(1000, 512, 1e-6, [
+    _lin(4, 128, 128, [0.9, 0.97, 0.99, 0.999]),
+    _att(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 256, ff=1024),
+    _ssm(16, 64, 128, 1, 4, 1),
+    _att(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 100, kv_from=1, ff=1024),
+])
+SEEDS = {"real": 16, "mix": 11, "att": 12, "ssm": 13, "lin": 14, "far": 15}
+PAGE = {"real": 16, "mix": 8, "att": 16, "ssm": 16, "lin": 8, "far": 16}
 SHARPEN = 3.0
 
 
@@ -235,6 +243,37 @@ def far_keys(env, name="far"):
     d.step({"r": ids[304:]})
     _check(env, folder, ids, d.result("w"), f"{name} whole")
     _check(env, folder, ids, d.result("r"), f"{name} cut around the block's edge")
+
+
+def real_sizes(env_f32, env_bf16, name="real"):
+    """At the layer sizes of a real model: float32 against the plain evaluation on a short prompt; then a prompt of 700
+    tokens (spans of the recurrence side by side, several blocks of both masks) whole, in portions and with its
+    last tokens decoded, bfloat16 against float32 of the same engine."""
+    page = PAGE[name]
+    V = _vocab(name)
+    short = random_ids(40, V, 900)
+    runner, manager, folder = env_f32.runner(name, 8, 1)
+    d = Driver(runner, manager)
+    d.step({"s": short[:33]})
+    d.step({"s": short[33:34]})
+    d.step({"s": short[34:]}, end=["s"])
+    _check(env_f32, folder, short, d.result("s"), f"{name} short prompt in float32")
+    n = 700
+    ids = random_ids(n, V, 901)
+    got = {}
+    for env in (env_f32, env_bf16):
+        runner, manager, folder = env.runner(name, 2 * -(-n // page), 2)
+        d = Driver(runner, manager)
+        d.step({"w": ids})
+        d.step({"r": ids[:300]})
+        d.step({"r": ids[300:302]})
+        d.step({"r": ids[302:680]})
+        for t in range(680, n):
+            d.step({"r": ids[t:t + 1]})
+        got[env.dtype] = (d.result("w"), d.result("r"))
+    (wf, rf), (wb, rb) = got[torch.float32], got[torch.bfloat16]
+    assert rel_err(rf, wf.double().cpu()) <= 1e-4, "float32: the cut request differs from the whole one"
+    assert rel_err(wb, wf.double().cpu()) <= env_bf16.tol and rel_err(rb, wf.double().cpu()) <= env_bf16.tol
 
 
 def slots_start_from_zero(env, name):

@@ -228,11 +228,11 @@ class Env:
     def runner(self, name, pages, slots):
         folder = self.folders(name)
         if name not in self.models:
-            self.models[name] = load_model(folder, self.device, self.dtype, 512)
+            self.models[name] = load_model(folder, self.device, self.dtype, 1024)
         model = self.models[name]
         manager = CacheManager(pages, S.PAGE[name], ModelRunner.windows_of(model), num_state_slots=slots, enable_prefix_caching=False)
         options = dict(use_graphs=True, mixed_graphs_after=1) if self.graphs else {}
-        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
+        return ModelRunner(model, manager, self.dtype, self.device, 1024, poison_cache=True, **options), manager, folder
 
 
 @pytest.fixture(scope="module", params=[torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
@@ -248,6 +248,10 @@ def test_cuts(env, case, name):
 
 def test_far_keys_and_block_edges(env):
     S.far_keys(env)
+
+
+def test_real_layer_sizes(sigosun_folders):
+    S.real_sizes(Env(sigosun_folders, torch.float32), Env(sigosun_folders, torch.bfloat16))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
