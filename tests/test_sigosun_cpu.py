@@ -101,3 +101,25 @@ def test_far_keys_and_block_edges(sigosun_folders, plain_backend):
 @pytest.mark.parametrize("name", ["mix", "lin"])
 def test_greedy_generation_through_the_scheduler(sigosun_folders, plain_backend, name):
     S.greedy_through_the_engine("cpu", "float32", name, sigosun_folders(name), exact=True)
+
+
+def test_command_line_on_a_folder_of_this_design(sigosun_folders, plain_backend, tmp_path, capsys):
+    """`python -m mini_engine_amd.cli --model DIR`: the folder's config picks the model class; prompts in, greedy tokens out."""
+    from mini_engine_amd import cli
+    import helpers
+    folder = sigosun_folders("mix")
+    prompts = [helpers.random_ids(n, 97, 950 + n) for n in (3, 19, 41)]
+    path = tmp_path / "prompts.jsonl"
+    path.write_text("\n".join(json.dumps(p) for p in prompts) + "\n")
+    out = tmp_path / "tokens.jsonl"
+    rc = cli.main(["--model", folder, "--prompts", str(path), "--tokens-out", str(out), "--temperature", "0", "--max-output", "6",
+                   "--dtype", "float32", "--device", "cpu", "--num-kv-blocks", "64", "--block-size", "8", "--budget", "16",
+                   "--max-num-seqs", "2", "--max-model-len", "128", "--out", str(tmp_path / "rows.jsonl")])
+    assert rc == 0
+    got = [json.loads(line) for line in open(out)]
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        assert len(g) == 6
+        for tok in g:
+            assert tok == int(S.plain_logits(folder, seq)[-1].argmax())
+            seq.append(tok)
