@@ -5,10 +5,11 @@ a block table per request, reference counts, chained xxh64 hashes of full pages 
 prefix reuse, oldest-freed-first recycling that evicts a page's hash when it is reused.
 Beyond it:
 
-* several **page groups**. Layers with different needs (all keys, or only a trailing
-  window of them) have pools and block tables of their own. In a window group the pages
-  that the window has passed are given back before new ones are taken; their table
-  entries become -1.
+* several **page groups**. Layers with different needs (all keys, only a trailing
+  window of them, or only the block of positions the next token falls into) have pools and
+  block tables of their own. In such a group the pages that the rule has passed are given
+  back before new ones are taken; their table entries become -1. A group's `window` is None,
+  an int (a window) or a tuple of rules (`first_kept`).
 * **state slots**: one slot per live request out of a fixed number, for mixers that
   keep state of fixed size. A request holds its slot from its first allocation to `free`.
 
@@ -38,6 +39,15 @@ def page_hash(token_ids, prefix: int = -1) -> int:
 class PrefixHit:
     num_pages: int = 0
     pages: list = field(default_factory=list)      # per group: page ids of the hit chain
+
+
+def first_kept(rule, num_computed: int) -> int:
+    """The first position whose keys a request still needs when its next token stands at `num_computed`. `rule`: an
+    int (a trailing window of that many positions) or a tuple of ("window", n) / ("chunk", c) rules, the loosest of
+    which holds; a chunk rule keeps the block of c positions, counted from 0, that `num_computed` falls into."""
+    if isinstance(rule, int):
+        return max(0, num_computed - rule + 1)
+    return min(max(0, num_computed - n + 1) if kind == "window" else (num_computed // n) * n for kind, n in rule)
 
 
 class _Group:
@@ -186,8 +196,8 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             if g.window is None:
                 continue
-            # the next tokens start at position num_computed and see keys >= num_computed - window + 1
-            first_needed = max(0, num_computed - g.window + 1)
+            # the next tokens start at position num_computed and see keys from first_kept on
+            first_needed = first_kept(g.window, num_computed)
             table = held.tables[gi]
             i = held.first_live[gi]
             while i < len(table) and (i + 1) * ps <= first_needed:

@@ -106,7 +106,7 @@ class ModelRunner:
     # -- sizing ----------------------------------------------------------------------------
     @staticmethod
     def windows_of(model) -> list:
-        return [need.window for need in model.cache_plan().group_needs]
+        return [need.keep() for need in model.cache_plan().group_needs]
 
     @staticmethod
     def pages_that_fit(model, page_size: int, dtype: torch.dtype, budget_bytes: int) -> int:

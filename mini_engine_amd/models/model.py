@@ -6,7 +6,7 @@ parameter is stored in a checkpoint (`weight_sources`).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 
 import torch
 
@@ -65,9 +65,16 @@ class DecoderModel(Part):
         keys: dict = {}
         needs, calls = [], []
         call_group, call_idx, call_writes, states = [], [], [], []
+        readers: dict = {}                 # owning call -> how long each call that reads its pages needs them
+        for call in self.order:
+            layer = self.layers[call.layer]
+            if call.cache_of is not None and hasattr(layer, "cache_need") and layer.cache_need() is not None:
+                readers.setdefault(call.cache_of, []).append(layer.cache_need().own_rule())
         for i, call in enumerate(self.order):
             layer = self.layers[call.layer]
             need: CacheNeed | None = layer.cache_need() if hasattr(layer, "cache_need") else None
+            if need is not None and i in readers:
+                need = replace(need, readers=tuple(readers[i]))
             state: StateNeed | None = layer.state_need() if hasattr(layer, "state_need") else None
             states.append(state)
             if need is None:

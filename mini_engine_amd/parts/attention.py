@@ -90,7 +90,7 @@ class Attention(Mixer):
             self.position = None
 
     def cache_need(self):
-        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window, self.chunk)
 
     def set_param(self, local, tensor):
         super().set_param(local, tensor)

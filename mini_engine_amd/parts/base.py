@@ -61,23 +61,45 @@ class PageTensor:
 class CacheNeed:
     """What a mixer wants from the paged cache: which tensors per token, and for how long.
 
-    ``window``: None keeps every token; n keeps the last n positions (pages that
-    the window has passed are given back). Layers with equal needs share one
+    ``window``: n keeps the last n positions; ``chunk``: c keeps the positions of the block of c
+    positions (counted from 0) that the next token falls into; neither: every token stays. Pages that
+    the rule has passed are given back. ``readers``: the rules of other layer calls that read these
+    pages (the model fills it in): the loosest of all rules holds. Layers with equal needs share one
     group of pages and one block table per request.
     """
 
     tensors: tuple                     # of PageTensor
     window: int | None = None
+    chunk: int | None = None
+    readers: tuple = ()                # own_rule() of every call that reads the pages of this one
 
     @classmethod
-    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int | None = None) -> "CacheNeed":
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int | None = None,
+                        chunk: int | None = None) -> "CacheNeed":
         """The layout of the attention kernels: K [pages, heads, page, head size], V [pages, heads, head
         size, page] (V transposed inside a page: the P.V operand of the matrix cores is then one load)."""
         return cls((PageTensor("k", (num_kv_heads, PAGE, head_dim)), PageTensor("v", (num_kv_heads, head_dim, PAGE))),
-                   window)
+                   window, chunk)
+
+    def own_rule(self) -> tuple:
+        """("window", n), ("chunk", c) or ("all", 0)."""
+        if self.window:
+            return ("window", int(self.window))
+        if self.chunk:
+            return ("chunk", int(self.chunk))
+        return ("all", 0)
+
+    def keep(self):
+        """What the cache manager is told: None (every token stays), an int (one trailing window), or a tuple of
+        ("window" | "chunk", n) rules of which the loosest holds at every moment."""
+        rules = {self.own_rule(), *self.readers}
+        if ("all", 0) in rules:
+            return None
+        rules = tuple(sorted(rules))
+        return rules[0][1] if len(rules) == 1 and rules[0][0] == "window" else rules
 
     def group_key(self) -> tuple:
-        return (self.tensors, self.window)
+        return (self.tensors, self.keep())
 
 
 @dataclass(frozen=True)

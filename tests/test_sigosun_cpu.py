@@ -76,6 +76,30 @@ def test_model_is_assembled_from_the_config():
     assert not any(n.startswith("l3.mix.k") or n.startswith("l3.mix.v") or n.startswith("l2.mlp") for n in names)
 
 
+def test_pages_behind_a_block_are_given_back():
+    """A block mask keeps the pages of the block the next token falls into; a group that another layer reads under a
+    mask of its own keeps what the loosest of the rules needs."""
+    from mini_engine_amd.cache.manager import first_kept
+    from mini_engine_amd.parts import CacheNeed
+    assert first_kept(5, 3) == 0 and first_kept(5, 12) == 8
+    assert [first_kept((("chunk", 7),), n) for n in (0, 6, 7, 13, 14)] == [0, 0, 7, 7, 14]
+    assert [first_kept((("chunk", 7), ("chunk", 10)), n) for n in (9, 10, 13, 14, 20, 21)] == [0, 7, 7, 10, 14, 20]
+    assert first_kept((("chunk", 8), ("window", 3)), 17) == 15
+    need = CacheNeed.keys_and_values(2, 16, chunk=7)
+    assert need.keep() == (("chunk", 7),) and CacheNeed.keys_and_values(2, 16, window=9).keep() == 9
+    assert CacheNeed.keys_and_values(2, 16).keep() is None
+    import dataclasses
+    assert dataclasses.replace(need, readers=(("chunk", 10),)).keep() == (("chunk", 7), ("chunk", 10))
+    assert dataclasses.replace(need, readers=(("all", 0),)).keep() is None          # a reader that sees every key
+    model = build_model(SigosunConfig.from_dict(S.CONFIGS["mix"]))
+    assert ModelRunner.windows_of(model) == [(("chunk", 7), ("chunk", 10))]
+    manager = CacheManager(8, 8, ModelRunner.windows_of(model), num_state_slots=1, enable_prefix_caching=False)
+    assert manager.allocate("r", 0, 30) and manager.block_table("r") == [0, 1, 2, 3]
+    assert manager.allocate("r", 30, 1) and manager.block_table("r") == [-1, -1, -1, 3]     # blocks start at 28 and 30: keys from 28 on
+    assert manager.allocate("r", 31, 10) and manager.block_table("r")[:3] == [-1, -1, -1] and manager.num_free_pages(0) == 5
+    manager.check_invariants()
+
+
 def test_head_order_of_rotations():
     assert RotaryEmbedding(16, 1e4).head_order() is None
     assert RotaryEmbedding(8, 1e4, interleaved=True).head_order() == [0, 2, 4, 6, 1, 3, 5, 7]
