@@ -66,12 +66,13 @@ def main(argv=None) -> int:
     tmp = None
     path = args.model
     if args.random_weights:
-        from .config.sizes import SIZES, model_config
+        from .config.sizes import SIZES, named_config
         from .weights.random_init import write_random_model
-        if args.random_weights not in SIZES:
-            p.error(f"--random-weights must be one of {sorted(SIZES)}")
+        try:
+            cfg, _ = named_config(args.random_weights)
+        except KeyError:
+            p.error(f"--random-weights must be one of {sorted(SIZES)}, or sigosun:<size> for that design at those layer sizes")
         tmp = tempfile.TemporaryDirectory()
-        cfg, _ = model_config(args.random_weights, None)
         path = write_random_model(cfg, args.seed, tmp.name)
     path = os.path.expanduser(path)
 

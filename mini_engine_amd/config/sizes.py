@@ -57,3 +57,12 @@ def sigosun_config(size: str, layers: int | None = None):
             out.append(attention(last_own))
     return SigosunConfig.from_dict({"architecture": "Sigosun", "vocab": V, "width": h, "norm": {"eps": 1e-6}, "layers": out,
                                     "max_position_embeddings": 40960}), L
+
+
+def named_config(name: str, layers: int | None = None):
+    """(configuration, full layer count) of a name the command lines take for random weights: a Qwen3 size
+    ("0.6b"), or "sigosun:<size>" for the Sigosun design at that size's layer sizes."""
+    design, _, size = name.rpartition(":")
+    if size not in SIZES or design not in ("", "qwen3", "sigosun"):
+        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:'")
+    return sigosun_config(size, layers) if design == "sigosun" else model_config(size, layers)

@@ -53,22 +53,22 @@ CONFIGS = {
     "mix": _model(97, 48, 1e-5, [
         _ssm(4, 12, 20, 2, 4, 2, ff=80),
         _att(4, 4, 24, 40, 0.3, 8, 5000.0, 7, ff=56),
-        _lin(3, 10, 20, [0.5, 0.93, 0.999]),
+        _lin(3, 10, 20, [0.5, 0.93, 0.998]),
         _att(4, 4, 24, 40, 0.2, 8, 5000.0, 10, kv_from=1),
         _ssm(2, 8, 16, 1, 2, 1),
     ]),
     # each mechanism alone
-    "att": _model(64, 32, 1e-6, [_att(6, 2, 16, 16, 0.25, 16, 10000.0, 5, ff=48)]),
+    "att": _model(64, 32, 1e-6, [_att(9, 3, 16, 16, 0.25, 16, 10000.0, 5, ff=48)]),
     "ssm": _model(64, 36, 1e-5, [_ssm(3, 80, 70, 1, 3, 1)]),          # value size above 64, state above 64 rows, a width that is no multiple of 8
     "lin": _model(64, 24, 1e-5, [_lin(2, 72, 8, [0.8, 0.9995])]),     # key size above 64: two slices of the state
     # long blocks: keys far back among hundreds; 1 key head for 3 query heads; key size 32 against value size 16
-    "far": _model(80, 32, 1e-5, [_att(3, 1, 32, 16, 0.2, 32, 250000.0, 300, ff=40), _lin(1, 16, 16, [0.999]),
-                                 _att(3, 1, 32, 16, 0.2, 32, 250000.0, 64, kv_from=0, ff=40)]),
+    "far": _model(80, 32, 1e-5, [_att(3, 1, 32, 16, 0.2, 32, 400000.0, 300, ff=40), _lin(1, 16, 16, [0.9985]),
+                                 _att(3, 1, 32, 16, 0.2, 32, 400000.0, 64, kv_from=0, ff=40)]),
 }
 # the layer sizes of a real model (heads of 128, a state of 128 x 64, four taps), few layers: the kernel forms that
 # the small widths above never reach
 CONFIGS["real"] = _model(1000, 512, 1e-6, [
-    _lin(4, 128, 128, [0.9, 0.97, 0.99, 0.999]),
+    _lin(4, 128, 128, [0.9, 0.97, 0.99, 0.9975]),
     _att(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 256, ff=1024),
     _ssm(16, 64, 128, 1, 4, 1),
     _att(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 100, kv_from=1, ff=1024),

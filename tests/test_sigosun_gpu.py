@@ -183,7 +183,7 @@ def test_attention_under_a_block_mask(dtype, chunk):
     """Prompts from their start, a portion behind a prefix and single tokens, at positions on both sides of block
     edges; one key per request is made to dominate, so a key wrongly seen or hidden shows."""
     torch.manual_seed(chunk)
-    Hq, Hkv, D, page = 6, 2, 64, 16
+    Hq, Hkv, D, page = 8, 2, 64, 16
     starts, q_lens = [chunk - 1, chunk, 2 * chunk + 3, 0, chunk - 3], [1, 1, 1, 2 * chunk + 9, 7]
     B, T = len(starts), sum(q_lens)
     ctx = [s + q for s, q in zip(starts, q_lens)]
@@ -209,7 +209,7 @@ def test_attention_under_a_block_mask(dtype, chunk):
     positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, q_lens)]).to(torch.int32).to(DEV)
     ctx_t = torch.tensor(ctx, dtype=torch.int32, device=DEV)
     prefill_cu = (cu[3:] - cu[3]).contiguous()
-    args = (q, k_cache, v_cache, page, bt, ctx_t, seq, positions, prefill_cu, 3, max(ctx[:3]), 0.125, None, Hq, Hkv, D)
+    args = (q, k_cache, v_cache, page, bt, ctx_t, seq, positions, prefill_cu, 3, max(ctx[:3]), 0.11, None, Hq, Hkv, D)
     got = hip().paged_attention(*args, max_prefill_context=max(ctx[3:]), chunk=chunk)
     want = twin.paged_attention(*args, chunk=chunk)
     close(got, want, 2e-5 if dtype == torch.float32 else 2e-2)
@@ -301,3 +301,18 @@ def test_trace_program_on_this_design(sigosun_folders, tmp_path, dtype):
     for r, g in TR.collect(steps, out, V).items():
         err = helpers.rel_err(g, S.plain_logits(folder, ids[r]))
         assert err <= TOL[getattr(torch, dtype)], f"{dtype} request {r}: {err:.3g}"
+
+
+def test_offline_workload_row_with_random_weights(tmp_path, capsys):
+    """The offline workload through the command line, on this design at a tiny size with random weights."""
+    import json
+    from mini_engine_amd import cli
+    rc = cli.main(["--random-weights", "sigosun:tinyA", "--num-seqs", "6", "--max-prompt", "40", "--max-output", "8",
+                   "--max-model-len", "64", "--max-num-seqs", "4", "--budget", "32", "--tokens-out", "-",
+                   "--out", str(tmp_path / "bench.jsonl")])
+    assert rc == 0
+    lines = capsys.readouterr().out.strip().splitlines()
+    row = json.loads(lines[-1])
+    tokens = [json.loads(line) for line in lines[-7:-1]]
+    assert [len(t) for t in tokens] == [8] * 6 and all(0 <= t < 256 for ts in tokens for t in ts)
+    assert row["num_seqs"] == 6 and row["output_tokens"] == 48 and row["throughput_tok_s"] > 0
