@@ -197,25 +197,40 @@ extern "C" int me_head_gate(void* o, const void* g, int64_t g_stride, int dtype,
 // request come from its state row: per channel taps - 1 values, oldest first. One thread per (token, channel).
 #define CONV_MAX_TAPS 16
 
+#define CONV_TOKENS 32       // tokens of one request that a thread walks
+
+// One thread per (request, block of CONV_TOKENS tokens, channel): it walks its tokens in order with the last taps - 1
+// inputs in registers, so every input is read once and the step's metadata once per workgroup.
 template <typename TX>
 __global__ void causal_conv_kernel(const TX* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                                    const float* __restrict__ bias, const float* __restrict__ state, int64_t state_stride,
                                    const int32_t* __restrict__ slots, const int32_t* __restrict__ cu,
-                                   const int32_t* __restrict__ seq_of_token, TX* __restrict__ out, int C, int taps) {
-  const int64_t t = blockIdx.x;
+                                   TX* __restrict__ out, int C, int taps, int blocks_per_seq) {
+  const int b = blockIdx.x / blocks_per_seq, blk = blockIdx.x - b * blocks_per_seq;
+  const int64_t first = cu[b];
+  const int n = (int)(cu[b + 1] - first);
+  const int l0 = blk * CONV_TOKENS;
+  if (l0 >= n) return;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
-  const int b = seq_of_token[t];
-  const int64_t first = cu[b];
-  const int local = (int)(t - first);
+  const int l1 = l0 + CONV_TOKENS < n ? l0 + CONV_TOKENS : n;
   const float* held = state + (int64_t)slots[b] * state_stride + (int64_t)c * (taps - 1);
-  float acc = bias[c];
-  for (int j = 0; j < taps; ++j) {
-    const int src = local - (taps - 1) + j;
-    const float v = src >= 0 ? to_f32<TX>(x[(first + src) * x_stride + c]) : held[src + taps - 1];
-    acc += w[(int64_t)c * taps + j] * v;
+  float wv[CONV_MAX_TAPS], seen[CONV_MAX_TAPS];
+  for (int j = 0; j < taps; ++j) wv[j] = w[(int64_t)c * taps + j];
+  // seen[j], j < taps - 1: the inputs at local positions l0 - (taps - 1) + j
+  for (int j = 0; j < taps - 1; ++j) {
+    const int src = l0 - (taps - 1) + j;
+    seen[j] = src >= 0 ? to_f32<TX>(x[(first + src) * x_stride + c]) : held[src + taps - 1];
   }
-  out[t * C + c] = from_f32<TX>(silu_f(acc));
+  const float bc = bias[c];
+  for (int l = l0; l < l1; ++l) {
+    const float now = to_f32<TX>(x[(first + l) * x_stride + c]);
+    float acc = bc + wv[taps - 1] * now;
+    for (int j = 0; j < taps - 1; ++j) acc += wv[j] * seen[j];
+    out[(first + l) * C + c] = from_f32<TX>(silu_f(acc));
+    for (int j = 0; j + 1 < taps - 1; ++j) seen[j] = seen[j + 1];
+    if (taps > 1) seen[taps - 2] = now;
+  }
 }
 
 // The state moves on: per (request, channel) the last taps - 1 inputs of (held inputs, this step's inputs).
@@ -257,8 +272,9 @@ __global__ void causal_conv_step_kernel(const TX* __restrict__ x, int64_t x_stri
   if (taps > 1) held[taps - 2] = now;
 }
 
+// max_tokens: no request brings more tokens than this.
 extern "C" int me_causal_conv(const void* x, int64_t x_stride, int dtype, const float* w, const float* bias, float* state,
-                              int64_t state_stride, const int32_t* slots, const int32_t* cu, const int32_t* seq_of_token,
+                              int64_t state_stride, const int32_t* slots, const int32_t* cu, int max_tokens,
                               void* out, int64_t T, int num_seqs, int C, int taps, hipStream_t stream) {
   if (T == 0 || C == 0) return 0;
   ME_CHECK(taps >= 1 && taps <= CONV_MAX_TAPS, "causal_conv: %d taps outside 1..%d", taps, CONV_MAX_TAPS);
@@ -276,12 +292,15 @@ extern "C" int me_causal_conv(const void* x, int64_t x_stride, int dtype, const 
     ME_LAUNCH_CHECK();
     return 0;
   }
+  const int blocks_per_seq = (max_tokens + CONV_TOKENS - 1) / CONV_TOKENS;
+  ME_CHECK(max_tokens >= 1 && (int64_t)num_seqs * blocks_per_seq <= 2147483647ll, "causal_conv: bad token bound %d", max_tokens);
+  const dim3 wgrid((unsigned)(num_seqs * blocks_per_seq), (C + block.x - 1) / block.x);
   if (dtype == ME_F32)
-    causal_conv_kernel<float><<<grid, block, 0, stream>>>((const float*)x, x_stride, w, bias, state, state_stride, slots, cu,
-                                                          seq_of_token, (float*)out, C, taps);
+    causal_conv_kernel<float><<<wgrid, block, 0, stream>>>((const float*)x, x_stride, w, bias, state, state_stride, slots, cu,
+                                                           (float*)out, C, taps, blocks_per_seq);
   else
-    causal_conv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, x_stride, w, bias, state, state_stride, slots, cu,
-                                                           seq_of_token, (bf16_t*)out, C, taps);
+    causal_conv_kernel<bf16_t><<<wgrid, block, 0, stream>>>((const bf16_t*)x, x_stride, w, bias, state, state_stride, slots, cu,
+                                                            (bf16_t*)out, C, taps, blocks_per_seq);
   ME_LAUNCH_CHECK();
   if (taps > 1) {
     const dim3 sgrid((C + block.x - 1) / block.x, num_seqs);

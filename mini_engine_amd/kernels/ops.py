@@ -74,7 +74,7 @@ _CORE_PROTOS = {
     "me_add_rms_norm_partials": [P, I, L, P, P, P, P, L, I, F, P],
     "me_activation": [P, L, P, I, I, L, I, P],
     "me_head_gate": [P, P, L, I, L, I, I, P],
-    "me_causal_conv": [P, L, I, P, P, P, L, P, P, P, P, L, I, I, I, P],
+    "me_causal_conv": [P, L, I, P, P, P, L, P, P, I, P, L, I, I, I, P],
     "me_linear_recurrence": [P, L, P, L, P, L, I, P, L, P, P, P, P, P, L, P, P, P, L, I, I, I, I, I, I, I, I, I, I, P, P],
     "me_gated_rms_norm": [P, I, L, P, L, I, P, P, L, I, I, I, F, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
@@ -613,11 +613,12 @@ class HipBackend:
         core().call("me_head_gate", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(o.dtype), T, H, D, _stream())
 
     # -- mixers with a state of fixed size -------------------------------------------------
-    def causal_conv(self, x, weight, bias, state, state_slots, cu_seqlens, seq_of_token) -> torch.Tensor:
+    def causal_conv(self, x, weight, bias, state, state_slots, cu_seqlens, q_lens) -> torch.Tensor:
         """silu(bias + sum_j weight[:, j] * x[t - (taps - 1) + j]) per channel over every request's tokens of this step,
         continued from its state: x a row view [T, C]; weight float32 [C, taps] (the last tap is the current
         token's); state a float32 view [slots, C * (taps - 1)] (per channel the inputs before the request's next
-        token, oldest first), rows `state_slots`; it moves on by this step's tokens. Returns [T, C]."""
+        token, oldest first), rows `state_slots`; it moves on by this step's tokens. `q_lens`: the requests' token
+        counts on the host (the launch is sized by the longest). Returns [T, C]."""
         T, C = x.shape
         taps = weight.shape[1]
         B = state_slots.numel()
@@ -625,10 +626,11 @@ class HipBackend:
                and bias.dtype == torch.float32 and bias.shape == (C,) and bias.is_contiguous(), "causal_conv: bad operands")
         _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] == C * (taps - 1),
                "causal_conv: state must be float32 [slots, C * (taps - 1)]")
-        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and _is_i32(seq_of_token, T), "causal_conv: metadata must be int32")
+        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B and sum(q_lens) == T,
+               "causal_conv: metadata must be int32, one token count per request")
         out = torch.empty((T, C), dtype=x.dtype, device=x.device)
         core().call("me_causal_conv", x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), bias.data_ptr(),
-                    state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_of_token.data_ptr(),
+                    state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), max(q_lens),
                     out.data_ptr(), T, B, C, taps, _stream())
         return out
 

@@ -114,7 +114,7 @@ class SelectiveStateSpace(Mixer):
         H, P, N, G = self.num_heads, self.value_dim, self.state_dim, self.groups
         rows = self.in_proj.forward(x)                                # [T, z | x | B | C | dt]
         xbc = ops.causal_conv(rows[:, self.inner: self.inner + self.channels], self.conv_weight, self.conv_bias,
-                              state[:, self.matrix_floats:], step.state_slots, step.cu_seqlens, step.seq_of_token)
+                              state[:, self.matrix_floats:], step.state_slots, step.cu_seqlens, step.q_lens)
         y = ops.linear_recurrence(xbc[:, self.inner + G * N:], xbc[:, self.inner: self.inner + G * N], xbc[:, : self.inner],
                                   state[:, : self.matrix_floats], step.state_slots, step.cu_seqlens, step.q_lens, H, G, N, P,
                                   dt=rows[:, self.inner + self.channels:], dt_bias=self.dt_bias, rate=self.rate, skip=self.D)

@@ -183,7 +183,7 @@ def head_gate(o, gate, H, D):
     o.copy_((o.float().view(T, H, D) * torch.sigmoid(gate.float())[:, :, None]).view(T, H * D).to(o.dtype))
 
 
-def causal_conv(x, weight, bias, state, state_slots, cu_seqlens, seq_of_token):
+def causal_conv(x, weight, bias, state, state_slots, cu_seqlens, q_lens):
     """x [T, C]; weight float32 [C, taps] (the last tap is the current token's), bias [C]; state [slots, C * (taps - 1)]
     float32: per channel the inputs before the request's next token, oldest first. silu(conv) in x's dtype; the state
     moves on."""

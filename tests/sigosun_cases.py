@@ -57,6 +57,14 @@ CONFIGS = {
         _att(4, 4, 24, 40, 0.2, 8, 5000.0, 10, kv_from=1),
         _ssm(2, 8, 16, 1, 2, 1),
     ]),
+    # attention first, its keys larger than its values, five query heads on one key head, an odd vocabulary; three groups
+    # and three norm groups; a feed-forward behind the linear attention; the reader's mask is the smaller one
+    "odd": _model(301, 72, 1e-6, [
+        _att(5, 1, 48, 32, 0.17, 16, 30000.0, 33),
+        _lin(2, 40, 24, [0.7, 0.99], ff=100),
+        _ssm(6, 20, 24, 3, 2, 3),
+        _att(5, 1, 48, 32, 0.21, 16, 30000.0, 9, kv_from=0, ff=64),
+    ]),
     # each mechanism alone
     "att": _model(64, 32, 1e-6, [_att(9, 3, 16, 16, 0.25, 16, 10000.0, 5, ff=48)]),
     "ssm": _model(64, 36, 1e-5, [_ssm(3, 80, 70, 1, 3, 1)]),          # value size above 64, state above 64 rows, a width that is no multiple of 8
@@ -73,8 +81,8 @@ CONFIGS["real"] = _model(1000, 512, 1e-6, [
     _ssm(16, 64, 128, 1, 4, 1),
     _att(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 100, kv_from=1, ff=1024),
 ])
-SEEDS = {"real": 16, "mix": 11, "att": 12, "ssm": 13, "lin": 14, "far": 15}
-PAGE = {"real": 16, "mix": 8, "att": 16, "ssm": 16, "lin": 8, "far": 16}
+SEEDS = {"real": 16, "odd": 17, "mix": 11, "att": 12, "ssm": 13, "lin": 14, "far": 15}
+PAGE = {"real": 16, "odd": 16, "mix": 8, "att": 16, "ssm": 16, "lin": 8, "far": 16}
 SHARPEN = 3.0
 
 

@@ -112,7 +112,7 @@ def test_head_order_of_rotations():
     assert abs(float(r.table[3, 1, 1]) - float(torch.sin(torch.tensor(3 * 100.0 ** -0.5, dtype=torch.float64)))) < 1e-7
 
 
-@pytest.mark.parametrize("name", ["mix", "att", "ssm", "lin"])
+@pytest.mark.parametrize("name", ["mix", "odd", "att", "ssm", "lin"])
 @pytest.mark.parametrize("case", S.ALL, ids=lambda c: c.__name__)
 def test_cuts(sigosun_folders, plain_backend, case, name):
     case(Env(sigosun_folders), name)

@@ -89,7 +89,7 @@ def test_causal_conv_continues_from_its_state(dtype, taps, C):
     """Requests of 1, 2, taps - 1, taps and many tokens in one step, each from a state of its own; then the same
     tokens cut in two steps give the same as in one."""
     torch.manual_seed(taps * C)
-    q_lens = [1, 2, max(1, taps - 1), taps, 37]
+    q_lens = [1, 2, max(1, taps - 1), taps, 77]
     cu, seq, slots = _steps_meta(q_lens, [3, 0, 5, 1, 2])
     T = sum(q_lens)
     rows = torch.randn(T, C + 9, device=DEV).to(dtype)
@@ -97,18 +97,18 @@ def test_causal_conv_continues_from_its_state(dtype, taps, C):
     w, b = torch.randn(C, taps, device=DEV), torch.randn(C, device=DEV)
     full = torch.randn(7, 11 + C * (taps - 1), device=DEV)
     st_h, st_t = full.clone(), full.clone()
-    got = hip().causal_conv(x, w, b, st_h[:, 11:], slots, cu, seq)
-    want = twin.causal_conv(x.cpu(), w.cpu(), b.cpu(), (st_c := st_t.cpu())[:, 11:], slots.cpu(), cu.cpu(), seq.cpu())
+    got = hip().causal_conv(x, w, b, st_h[:, 11:], slots, cu, q_lens)
+    want = twin.causal_conv(x.cpu(), w.cpu(), b.cpu(), (st_c := st_t.cpu())[:, 11:], slots.cpu(), cu.cpu(), q_lens)
     close(got, want, 1e-6 if dtype == torch.float32 else 8e-3)
     close(st_h, st_c, 1e-6)
     assert torch.equal(st_h[:, :11], full[:, :11]) and torch.equal(st_h[4], full[4]) and torch.equal(st_h[6], full[6])
-    # the last request again, cut after 5 tokens
+    # the last request again (77 tokens: three blocks of a thread's 32), cut after 5 tokens
     st2 = full.clone()
     cu1, seq1, sl1 = _steps_meta([5], [2])
-    first = hip().causal_conv(x[T - 37:T - 32], w, b, st2[:, 11:], sl1, cu1, seq1)
-    cu2, seq2, _ = _steps_meta([32], [2])
-    rest = hip().causal_conv(x[T - 32:], w, b, st2[:, 11:], sl1, cu2, seq2)
-    assert torch.equal(torch.cat((first, rest)), got[T - 37:]) and torch.equal(st2[2], st_h[2])
+    first = hip().causal_conv(x[T - 77:T - 72], w, b, st2[:, 11:], sl1, cu1, [5])
+    cu2, seq2, _ = _steps_meta([72], [2])
+    rest = hip().causal_conv(x[T - 72:], w, b, st2[:, 11:], sl1, cu2, [72])
+    assert torch.equal(torch.cat((first, rest)), got[T - 77:]) and torch.equal(st2[2], st_h[2])
 
 
 @pytest.mark.parametrize("columns", [1, 2])
@@ -240,7 +240,7 @@ def env(request, sigosun_folders):
     return Env(sigosun_folders, request.param)
 
 
-@pytest.mark.parametrize("name", ["mix", "att", "ssm", "lin"])
+@pytest.mark.parametrize("name", ["mix", "odd", "att", "ssm", "lin"])
 @pytest.mark.parametrize("case", S.ALL, ids=lambda c: c.__name__)
 def test_cuts(env, case, name):
     case(env, name)
