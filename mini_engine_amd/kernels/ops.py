@@ -668,7 +668,7 @@ class HipBackend:
         per_wave = recurrence_rows_per_wave(N)
         slices = -(-N // per_wave)
         columns = recurrence_columns(q_lens, H, G, P, slices)
-        span, spans = recurrence_spans(q_lens, H * -(-P // 64) * slices // columns)
+        span, spans = recurrence_spans(q_lens, H * -(-P // 64) * slices // columns, 65535 // slices)
         scratch = _scratch(B * spans * (H * N * P + H), v.device, "recurrence") if spans > 1 else None
         y = torch.empty((slices, T, H * P) if slices > 1 else (T, H * P), dtype=torch.float32, device=v.device)
         core().call("me_linear_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
@@ -1134,7 +1134,7 @@ RECURRENCE_MIN_SPAN = 64
 RECURRENCE_WAVES = 4096        # waves that keep the 256 compute units busy: 16 a unit, 4 a SIMD
 
 
-def recurrence_spans(q_lens: list, waves_per_request: int) -> tuple:
+def recurrence_spans(q_lens: list, waves_per_request: int, most_spans: int = 8191) -> tuple:
     """(tokens per span, most spans per request) for the recurrence kernel; (0, 1): every request in one pass.
 
     A request's tokens are a chain, and one pass gives the GPU only requests x heads x slices waves. A long prompt is
@@ -1148,7 +1148,7 @@ def recurrence_spans(q_lens: list, waves_per_request: int) -> tuple:
         return 0, 1
     total = sum(q_lens)
     want = max(1, RECURRENCE_WAVES // max(1, waves_per_request))        # spans over all requests
-    span = max(RECURRENCE_MIN_SPAN, -(-total // want))
+    span = max(RECURRENCE_MIN_SPAN, -(-total // want), -(-longest // most_spans))    # a launch holds `most_spans` spans a request
     span = -(-span // 16) * 16
     spans = -(-longest // span)
     return (span, spans) if spans >= 2 else (0, 1)

@@ -147,3 +147,23 @@ def test_command_line_on_a_folder_of_this_design(sigosun_folders, plain_backend,
         for tok in g:
             assert tok == int(S.plain_logits(folder, seq)[-1].argmax())
             seq.append(tok)
+
+
+def test_launch_rules_of_the_recurrence():
+    """Whatever the step, the spans cover the longest request, keep 64 tokens or more in whole batches of the kernel's 8,
+    and stay within one launch; the rows a wave keeps are a size the kernel is built for and cover N."""
+    from mini_engine_amd.kernels import ops
+    import random
+    rng = random.Random(0)
+    for _ in range(2000):
+        q_lens = [rng.choice((1, 2, 17, 63, 64, 127, 128, 129, 700, 5000, 40000)) for _ in range(rng.randint(1, 40))]
+        waves = rng.choice((1, 4, 64, 128, 1024))
+        span, spans = ops.recurrence_spans(q_lens, waves)
+        if spans == 1:
+            assert span == 0 and (max(q_lens) < 128 or -(-sum(q_lens) // max(1, 4096 // waves)) >= max(q_lens))
+        else:
+            assert span >= 64 and span % 8 == 0 and spans * span >= max(q_lens) and (spans - 1) * span < max(q_lens)
+            assert spans * 4 <= 65535
+    for N in list(range(1, 300)) + [512, 1000, 4096]:
+        rows = ops.recurrence_rows_per_wave(N)
+        assert rows in (16, 32, 48, 64) and -(-N // rows) * rows >= N and -(-N // rows) * rows - N < rows
