@@ -10,6 +10,7 @@
 //
 // Everything that enters a recurrence is float32: step sizes, decays, their exponentials, the state, the sums.
 #include "common.h"
+#include <type_traits>
 
 #define RC_MAX_PARTIALS 8
 
@@ -349,7 +350,8 @@ template <typename TX, int NT, int PASS, int HPB, int PPB>
 __global__ void __launch_bounds__(64) recurrence_kernel(RecArgs a) {
   constexpr int CL = HPB * PPB;
   constexpr int KR = REC_TB * NT / 64;               // k (and q) values a lane carries to LDS per batch of tokens
-  __shared__ float2 skq[REC_TB][NT];
+  using Cell = std::conditional_t<PASS == 1, float, float2>;       // the first pass of spans reads no q
+  __shared__ Cell skq[REC_TB][NT];
   __shared__ float sa[HPB][REC_TB], sb[HPB][REC_TB];
   const int lane = threadIdx.x;
   const int heads_blocks = a.H / HPB;
@@ -459,7 +461,8 @@ __global__ void __launch_bounds__(64) recurrence_kernel(RecArgs a) {
       const int i = lane + r * 64, tt = i / NT, nn = i - tt * NT;
       float kk = kreg[r], qq = PASS != 1 ? qreg[r] : 0.f;
       if (silu) { kk = silu_f(kk); qq = silu_f(qq); }
-      skq[tt][nn] = make_float2(kk, qq);
+      if constexpr (PASS == 1) skq[tt][nn] = kk;
+      else skq[tt][nn] = make_float2(kk, qq);
     }
     if (lane < HPB * REC_TB) { sa[lane / REC_TB][lane % REC_TB] = areg; sb[lane / REC_TB][lane % REC_TB] = breg; }
 #pragma unroll
@@ -481,11 +484,17 @@ __global__ void __launch_bounds__(64) recurrence_kernel(RecArgs a) {
       }
 #pragma unroll
       for (int i = 0; i < NT; ++i) {
-        const float2 kq = skq[tt][i];
+        if constexpr (PASS == 1) {
+          const float kk = skq[tt][i];
 #pragma unroll
-        for (int j = 0; j < CL; ++j) {
-          S[j][i] = da[j] * S[j][i] + kq.x * bv[j];
-          if (PASS != 1) acc[j] += S[j][i] * kq.y;
+          for (int j = 0; j < CL; ++j) S[j][i] = da[j] * S[j][i] + kk * bv[j];
+        } else {
+          const float2 kq = skq[tt][i];
+#pragma unroll
+          for (int j = 0; j < CL; ++j) {
+            S[j][i] = da[j] * S[j][i] + kq.x * bv[j];
+            acc[j] += S[j][i] * kq.y;
+          }
         }
       }
       if (PASS == 1) {
