@@ -377,3 +377,147 @@ class SigosunConfig:
     def flat(self) -> dict[str, Any]:
         return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
                 "layer_kinds": [layer.kind for layer in self.layers]}
+
+
+# ------------------------------------------------------------------------------------ Negosun
+
+@dataclass(frozen=True)
+class NegosunLayer:
+    """One entry of a Negosun config's `layers`: the mixer's sizes and constants (validated, optional keys resolved)
+    and the feed-forward's (None: the layer has no feed-forward)."""
+
+    kind: str                  # "attention"
+    mixer: dict
+    mlp: dict | None
+
+
+@register_config("Negosun")
+@dataclass(frozen=True)
+class NegosunConfig:
+    """The ``config.json`` keys of the Negosun design: layers whose mixer and feed-forward read the same stream side by
+    side, each through a norm of its own, their outputs scaled element by element and added under one multiplier
+    (`residual_mult`); attention with biases, q and k normed over the whole projection, a query temperature that grows
+    with the logarithm of the position, and values blended with those of the first such layer (`v_mix`); a
+    feed-forward of routed experts with an optional limit to the best groups and an optional shared expert; tied
+    output weights and an optional soft cap on the logits. Every size and constant comes from the file."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    residual_mult: float
+    logit_softcap: float | None
+    layers: tuple
+    eos_token_id: int | None = None
+    max_position_embeddings: int | None = None
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict[str, Any]) -> "NegosunConfig":
+        norm = raw.get("norm")
+        if not isinstance(norm, dict):
+            raise ConfigError("config.json lacks the object 'norm'")
+        listed = raw.get("layers")
+        if not isinstance(listed, list) or not listed:
+            raise ConfigError("config.json lacks the list 'layers'")
+        layers = []
+        for i, entry in enumerate(listed):
+            where = f"layers[{i}]"
+            kind = entry.get("type") if isinstance(entry, dict) else None
+            if kind != "attention":
+                raise ConfigError(f"{where}: 'type' must be 'attention', got {kind!r}")
+            m = entry.get("mixer")
+            if not isinstance(m, dict):
+                raise ConfigError(f"{where} lacks the object 'mixer'")
+            mixer = {key: _need(m, key, typ, where + ".mixer")
+                     for key, typ in (("heads", int), ("kv_heads", int), ("dim", int), ("vdim", int), ("scale", float))}
+            temp = m.get("q_temp")
+            mixer["temp_coef"] = _need(temp, "coef", float, where + ".mixer.q_temp") if temp else None
+            mixer["temp_every"] = _need(temp, "every", int, where + ".mixer.q_temp") if temp else None
+            mixer["v_mix"] = bool(m.get("v_mix", False))
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                if mlp.get("kind", "moe") != "moe":
+                    raise ConfigError(f"{where}.mlp: only kind 'moe' is known, got {mlp.get('kind')!r}")
+                router = mlp.get("router")
+                if not isinstance(router, dict) or not isinstance(mlp.get("expert"), dict):
+                    raise ConfigError(f"{where}.mlp lacks the objects 'router' and 'expert'")
+                groups, shared = router.get("groups"), mlp.get("shared")
+                ff = {"ff": _need(mlp["expert"], "ff", int, where + ".mlp.expert"),
+                      "experts": _need(router, "experts", int, where + ".mlp.router"),
+                      "top": _need(router, "top", int, where + ".mlp.router"),
+                      "group_count": _need(groups, "count", int, where + ".mlp.router.groups") if groups else 1,
+                      "group_keep": _need(groups, "keep", int, where + ".mlp.router.groups") if groups else 1,
+                      "shared_ff": _need(shared, "ff", int, where + ".mlp.shared") if shared else None}
+            layers.append(NegosunLayer(kind, mixer, ff))
+        cap = raw.get("logit_softcap")
+        cfg = cls(vocab_size=_need(raw, "vocab", int), hidden_size=_need(raw, "width", int),
+                  norm_eps=_need(norm, "eps", float, "config.json norm"),
+                  residual_mult=float(raw["residual_mult"]) if raw.get("residual_mult") is not None else 1.0,
+                  logit_softcap=None if cap is None else float(cap), layers=tuple(layers),
+                  eos_token_id=raw.get("eos_token_id"), max_position_embeddings=raw.get("max_position_embeddings"))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.norm_eps > 0:
+            raise ConfigError("vocab and width must be positive and norm.eps above zero")
+        if self.logit_softcap is not None and not self.logit_softcap > 0:
+            raise ConfigError("logit_softcap must be positive")
+        mixed = None
+        for i, layer in enumerate(self.layers):
+            m, where = layer.mixer, f"layers[{i}]"
+            if any(m[k] < 1 for k in ("heads", "kv_heads", "dim", "vdim")):
+                raise ConfigError(f"{where}: sizes must be positive")
+            if m["heads"] % m["kv_heads"]:
+                raise ConfigError(f"{where}: {m['heads']} heads are not a multiple of {m['kv_heads']} kv_heads")
+            if m["temp_every"] is not None and m["temp_every"] < 1:
+                raise ConfigError(f"{where}: q_temp.every must be positive")
+            if m["v_mix"]:
+                width = m["kv_heads"] * m["vdim"]
+                if mixed is not None and width != mixed:
+                    raise ConfigError(f"{where}: layers with v_mix must have equally many value dimensions ({width} against {mixed})")
+                mixed = width
+            f = layer.mlp
+            if f is not None:
+                if f["ff"] < 1 or f["experts"] < 1 or not 1 <= f["top"] <= f["experts"]:
+                    raise ConfigError(f"{where}.mlp: sizes must be positive and top at most experts")
+                if f["group_count"] < 1 or f["experts"] % f["group_count"] or not 1 <= f["group_keep"] <= f["group_count"]:
+                    raise ConfigError(f"{where}.mlp: {f['experts']} experts do not form {f['group_count']} equal groups "
+                                      f"of which {f['group_keep']} are kept")
+                if f["group_keep"] * (f["experts"] // f["group_count"]) < f["top"]:
+                    raise ConfigError(f"{where}.mlp: the kept groups hold fewer experts than a token uses")
+                if f["shared_ff"] is not None and f["shared_ff"] < 1:
+                    raise ConfigError(f"{where}.mlp.shared: ff must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        """A ``config.json`` that reads back to an equal config."""
+        out = []
+        for layer in self.layers:
+            m = {k: layer.mixer[k] for k in ("heads", "kv_heads", "dim", "vdim", "scale", "v_mix")}
+            if layer.mixer["temp_every"] is not None:
+                m["q_temp"] = {"coef": layer.mixer["temp_coef"], "every": layer.mixer["temp_every"]}
+            f = layer.mlp
+            mlp = None
+            if f is not None:
+                mlp = {"kind": "moe", "expert": {"ff": f["ff"]},
+                       "router": {"experts": f["experts"], "top": f["top"], "groups": {"count": f["group_count"], "keep": f["group_keep"]}}}
+                if f["shared_ff"] is not None:
+                    mlp["shared"] = {"ff": f["shared_ff"]}
+            out.append({"type": layer.kind, "mixer": m, "mlp": mlp})
+        d = {"architecture": self.architecture_name, "vocab": self.vocab_size, "width": self.hidden_size,
+             "norm": {"eps": self.norm_eps}, "residual_mult": self.residual_mult, "layers": out}
+        if self.logit_softcap is not None:
+            d["logit_softcap"] = self.logit_softcap
+        if self.eos_token_id is not None:
+            d["eos_token_id"] = self.eos_token_id
+        if self.max_position_embeddings is not None:
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d
+
+    def flat(self) -> dict[str, Any]:
+        return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
+                "experts": [None if layer.mlp is None else layer.mlp["experts"] for layer in self.layers]}

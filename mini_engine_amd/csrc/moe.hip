@@ -1,0 +1,413 @@
+// A feed-forward made of many small gated experts of which every token uses a few.
+//
+//   moe_route      float32 router: logits = W x, softmax over all experts, optionally only the experts of the best
+//                  groups of neighbours stay eligible (a group scores as its best expert), the `top` largest scores
+//                  are chosen and divided by their sum
+//   moe_sort       (token, choice) pairs ordered by expert, cut into tiles of 64 rows that never span two experts
+//   moe_gate_up    per tile: silu(x W_gate^T) * (x W_up^T) of the tile's expert, token rows gathered through the order
+//   moe_down       per tile: the expert's down product, times the pair's weight, into float32 [top, T, hidden]: one
+//                  partial sum per choice, for a consumer that adds them (no atomics: the result does not depend on
+//                  what else is in the batch)
+//   moe_*_simple   the same two products with one wave per output element: the float32 path, and sizes whose rows
+//                  are not whole 16-byte pieces
+//
+// The tiled kernels: a workgroup owns 64 pair rows x 64 weight rows, its 4 waves 2 x 2 sub-tiles of 32 x 32
+// (v_mfma_f32_16x16x32_bf16, weight rows as the A operand, so that a lane holds 4 consecutive features of one
+// row); K is walked 64 at a time through two LDS buffers, the next step's 16-byte pieces on their way in registers
+// while the current one is multiplied; piece c of row R lies at c ^ (R >> 1 & 7), so that the 16 lanes of an operand
+// read touch 16 different bank groups. Pieces beyond K are zeros, so K needs to be a multiple of 8 only.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_TM 64
+
+// ------------------------------------------------------------------ router
+// Orders a wave's LDS writes before its later reads of them by other lanes.
+__device__ __forceinline__ void wave_settle() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off, ME_WAVE);
+    const int oi = __shfl_xor(i, off, ME_WAVE);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+}
+
+// One workgroup of 4 waves per `tokens_per_group` tokens (their rows wait in LDS); a wave takes every fourth expert's
+// dot products, then every fourth token's selection. LDS: rows, then per token E scores, E working copies, and the
+// group scores.
+template <typename TX>
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t T, int n, int E, int top,
+                 int group_count, int group_keep, int tokens_per_group, int32_t* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ __align__(16) unsigned char route_lds[];
+  const int TT = tokens_per_group;
+  TX* xs = reinterpret_cast<TX*>(route_lds);
+  float* score = reinterpret_cast<float*>(route_lds + (((size_t)TT * n * sizeof(TX) + 15) & ~(size_t)15));
+  float* work = score + (size_t)TT * E;
+  float* gscore = work + (size_t)TT * E;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t0 = (int64_t)blockIdx.x * TT;
+  const int live = (int)min((int64_t)TT, T - t0);
+  for (int i = threadIdx.x; i < TT * n; i += blockDim.x) {
+    const int tt = i / n, k = i - tt * n;
+    xs[i] = tt < live ? x[(t0 + tt) * ldx + k] : from_f32<TX>(0.f);
+  }
+  __syncthreads();
+  for (int e = wave; e < E; e += 4) {
+    float acc[8];
+#pragma unroll
+    for (int tt = 0; tt < 8; ++tt) acc[tt] = 0.f;
+    const float* we = w + (int64_t)e * n;
+    for (int k = lane; k < n; k += 64) {
+      const float wv = we[k];
+#pragma unroll
+      for (int tt = 0; tt < 8; ++tt)
+        if (tt < TT) acc[tt] += wv * to_f32<TX>(xs[tt * n + k]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < 8; ++tt)
+      if (tt < TT) {
+        const float s = wave_sum(acc[tt]);
+        if (lane == 0) score[tt * E + e] = s;
+      }
+  }
+  __syncthreads();
+  const int per = E / group_count;
+  for (int tt = wave; tt < live; tt += 4) {
+    float* s = score + tt * E;
+    float* m = work + tt * E;
+    float* gs = gscore + tt * group_count;
+    float hi = -INFINITY;
+    for (int e = lane; e < E; e += 64) hi = fmaxf(hi, s[e]);
+    hi = wave_max(hi);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) { const float p = expf(s[e] - hi); s[e] = p; sum += p; }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) { s[e] = s[e] / sum; m[e] = s[e]; }
+    wave_settle();
+    if (group_count > 1 && group_keep < group_count) {
+      for (int g = lane; g < group_count; g += 64) {
+        float best = -1.f;
+        for (int j = 0; j < per; ++j) best = fmaxf(best, s[g * per + j]);
+        gs[g] = best;
+      }
+      wave_settle();
+      // the best groups one after the other; a kept group's score drops to -2, the others' experts leave the race
+      for (int kept = 0; kept < group_keep; ++kept) {
+        float bv = -3.f; int bi = 0x7fffffff;
+        for (int g = lane; g < group_count; g += 64)
+          if (gs[g] > bv) { bv = gs[g]; bi = g; }
+        wave_argmax(bv, bi);
+        if (bi >= group_count) bi = 0;          // scores that are no numbers: still a valid index
+        if (lane == 0) gs[bi] = -2.f;
+        wave_settle();
+      }
+      for (int e = lane; e < E; e += 64)
+        if (gs[e / per] != -2.f) m[e] = -1.f;
+      wave_settle();
+    }
+    float total = 0.f;
+    int mine = -1;           // lane j keeps the j-th choice (top <= 64)
+    for (int j = 0; j < top; ++j) {
+      float bv = -3.f; int bi = 0x7fffffff;
+      for (int e = lane; e < E; e += 64)
+        if (m[e] > bv) { bv = m[e]; bi = e; }
+      wave_argmax(bv, bi);
+      if (bi >= E) bi = 0;
+      if (lane == 0) m[bi] = -2.f;
+      wave_settle();
+      if (lane == j) mine = bi;
+      total += s[bi];
+    }
+    if (lane < top) {
+      ids[(t0 + tt) * top + lane] = mine;
+      weights[(t0 + tt) * top + lane] = s[mine] / (total + 1e-20f);
+    }
+  }
+}
+
+extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* w, int64_t T, int n, int E, int top,
+                            int group_count, int group_keep, int32_t* ids, float* weights, hipStream_t stream) {
+  if (T == 0) return 0;
+  ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && top >= 1 && top <= 64 && top <= E, "moe_route: %d experts, top %d", E, top);
+  ME_CHECK(group_count >= 1 && E % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+           "moe_route: %d groups (keep %d) over %d experts", group_count, group_keep, E);
+  ME_CHECK(group_keep * (E / group_count) >= top, "moe_route: the kept groups hold fewer than top experts");
+  const size_t es = dtype == ME_F32 ? 4 : 2;
+  int TT = 8;
+  while (TT > 1 && (size_t)TT * n * es > 32 * 1024) TT >>= 1;
+  const size_t lds = (((size_t)TT * n * es + 15) & ~(size_t)15) + (size_t)TT * (2 * E + group_count) * 4;
+  ME_CHECK(lds <= 64 * 1024, "moe_route: width %d with %d experts does not fit a workgroup's memory", n, E);
+  const int64_t groups = (T + TT - 1) / TT;
+  ME_CHECK(groups < (1ll << 31), "moe_route: too many tokens");
+  if (dtype == ME_F32)
+    moe_route_kernel<float><<<dim3((unsigned)groups), dim3(256), lds, stream>>>((const float*)x, ldx, w, T, n, E, top, group_count,
+                                                                                group_keep, TT, ids, weights);
+  else
+    moe_route_kernel<bf16_t><<<dim3((unsigned)groups), dim3(256), lds, stream>>>((const bf16_t*)x, ldx, w, T, n, E, top, group_count,
+                                                                                 group_keep, TT, ids, weights);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ pairs by expert
+// One workgroup. order[p']: the pair at sorted place p'; offsets[e]: where expert e's pairs begin; tile_expert / tile_row:
+// expert and first sorted place of every tile of up to 64 pairs (expert -1: a tile nobody needs).
+__global__ void __launch_bounds__(1024)
+moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, int32_t* __restrict__ order,
+                int32_t* __restrict__ offsets, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row) {
+  __shared__ int count[MOE_MAX_EXPERTS], begin[MOE_MAX_EXPERTS + 1], tile_at[MOE_MAX_EXPERTS + 1], cursor[MOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      begin[e] = at; tile_at[e] = tiles;
+      at += count[e];
+      tiles += (count[e] + MOE_TM - 1) / MOE_TM;
+    }
+    begin[E] = at; tile_at[E] = tiles;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = begin[e];
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids[p];
+    order[begin[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+  for (int e = threadIdx.x; e < E; e += blockDim.x)
+    for (int i = tile_at[e]; i < tile_at[e + 1] && i < max_tiles; ++i) {
+      tile_expert[i] = e;
+      tile_row[i] = begin[e] + (i - tile_at[e]) * MOE_TM;
+    }
+  for (int i = tile_at[E] + threadIdx.x; i < max_tiles; i += blockDim.x) { tile_expert[i] = -1; tile_row[i] = 0; }
+}
+
+extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, int32_t* order, int32_t* offsets,
+                           int32_t* tile_expert, int32_t* tile_row, hipStream_t stream) {
+  if (P == 0) return 0;
+  ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && P < (1ll << 30), "moe_sort: %d experts, %lld pairs", E, (long long)P);
+  ME_CHECK(max_tiles >= P / MOE_TM + (P < E ? P : E), "moe_sort: %d tiles cannot hold every expert's last tile", max_tiles);
+  moe_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, (int)P, E, max_tiles, order, offsets, tile_expert, tile_row);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ tiled products
+// A stage in LDS: 64 B rows (pairs) then 64 A rows (weights), 128 bytes each.
+struct MoeStage {
+  uint4 piece[4];
+};
+
+// ACT: the tile's weight rows are 32 gate rows and the 32 up rows that go with them; the result is silu(gate) * up.
+//   x: [T, K] token rows (ACT) or [P, K] rows at sorted places; w: [E * rows_per_expert, K]
+template <bool ACT>
+__global__ void __launch_bounds__(256)
+moe_tile_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
+                const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const int32_t* __restrict__ tile_expert,
+                const int32_t* __restrict__ tile_row, const float* __restrict__ pair_weight, void* __restrict__ out,
+                int64_t T, int top, int N, int K) {
+  __shared__ __align__(16) unsigned char lds[2][128 * 128];
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int row0 = tile_row[blockIdx.y];
+  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (ACT ? 32 : 64);           // first feature of the tile
+  // the 4 pieces this thread brings per stage: rows tid / 8 + 32 q, piece tid % 8
+  const bf16_t* src[4];
+  uint32_t dst[4];
+  const int c = tid & 7;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int R = (tid >> 3) + 32 * q;
+    if (R < MOE_TM) {
+      const int p = row0 + min(R, rows - 1);
+      const int64_t from = ACT ? (int64_t)(order[p] / top) : (int64_t)p;
+      src[q] = x + from * ldx;
+    } else {
+      const int wr = R - MOE_TM;
+      int64_t row;
+      if (ACT) row = (int64_t)e * 2 * N + (wr < 32 ? min(n0 + wr, N - 1) : N + min(n0 + wr - 32, N - 1));
+      else row = (int64_t)e * N + min(n0 + wr, N - 1);
+      src[q] = w + row * ldw;
+    }
+    dst[q] = R * 128 + ((c ^ ((R >> 1) & 7)) * 16);
+  }
+  auto fetch = [&](int k0, MoeStage& st) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int k = k0 + 8 * c;
+      st.piece[q] = k < K ? *reinterpret_cast<const uint4*>(src[q] + k) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  auto put = [&](int b, const MoeStage& st) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4*>(&lds[b][dst[q]]) = st.piece[q];
+  };
+  const int wm = wave >> 1, wn = wave & 1;
+  const int swz = (n >> 1) & 7;
+  uint32_t rd_b[2], rd_a[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    rd_b[s] = (wm * 32 + n) * 128 + (((4 * s + g) ^ swz) * 16);
+    rd_a[s] = (MOE_TM + wn * (ACT ? 16 : 32) + n) * 128 + (((4 * s + g) ^ swz) * 16);
+  }
+  f32x4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (K + 63) / 64;
+  MoeStage st;
+  fetch(0, st);
+  put(0, st);
+  __syncthreads();
+  for (int k = 0; k < steps; ++k) {
+    if (k + 1 < steps) fetch((k + 1) * 64, st);
+    const unsigned char* buf = lds[k & 1];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + (ACT ? 32 : 16) * 128 * i);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + rd_b[s] + 16 * 128 * j);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (k + 1 < steps) put((k + 1) & 1, st);
+    __syncthreads();
+  }
+  // lane (n, g) of tile (i, j): features ... + 4 g .. + 3 of pair row 32 wm + 16 j + n
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int r = wm * 32 + 16 * j + n;
+    if (r >= rows) continue;
+    const int p = row0 + r;
+    if constexpr (ACT) {
+      bf16_t* o = (bf16_t*)out + (int64_t)p * N;
+      const int f = n0 + wn * 16 + 4 * g;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (f + q < N) {
+          const float gate = acc[0][j][q];
+          o[f + q] = from_f32<bf16_t>(gate / (1.f + __expf(-gate)) * acc[1][j][q]);
+        }
+    } else {
+      const int pair = order[p];
+      const int64_t tok = pair / top, choice = pair - tok * top;
+      const float pw = pair_weight[pair];
+      float* o = (float*)out + (choice * T + tok) * N;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int f = n0 + wn * 32 + 16 * i + 4 * g;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (f + q < N) o[f + q] = acc[i][j][q] * pw;
+      }
+    }
+  }
+}
+
+// act: bfloat16 [P, F] at sorted places; gate_up: [E * 2 F, K] (an expert's gate rows, then its up rows)
+extern "C" int me_moe_gate_up(const void* x, int64_t ldx, const void* gate_up, const int32_t* order, const int32_t* offsets,
+                              const int32_t* tile_expert, const int32_t* tile_row, void* act, int64_t T, int top, int F, int K,
+                              int max_tiles, hipStream_t stream) {
+  if (T == 0) return 0;
+  ME_CHECK(K % 8 == 0 && ldx % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0,
+           "moe_gate_up: rows must be whole 16-byte pieces (K = %d)", K);
+  ME_CHECK(max_tiles >= 1 && max_tiles <= 65535 && F >= 1, "moe_gate_up: %d tiles", max_tiles);
+  moe_tile_kernel<true><<<dim3((unsigned)((F + 31) / 32), (unsigned)max_tiles), dim3(256), 0, stream>>>(
+      (const bf16_t*)x, ldx, (const bf16_t*)gate_up, (int64_t)K, order, offsets, tile_expert, tile_row, nullptr, act, T, top, F, K);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// out: float32 [top, T, N]; down: [E * N, F]
+extern "C" int me_moe_down(const void* act, const void* down, const int32_t* order, const int32_t* offsets,
+                           const int32_t* tile_expert, const int32_t* tile_row, const float* pair_weight, float* out, int64_t T,
+                           int top, int N, int F, int max_tiles, hipStream_t stream) {
+  if (T == 0) return 0;
+  ME_CHECK(F % 8 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0 && reinterpret_cast<uintptr_t>(down) % 16 == 0,
+           "moe_down: rows must be whole 16-byte pieces (F = %d)", F);
+  ME_CHECK(max_tiles >= 1 && max_tiles <= 65535 && N >= 1, "moe_down: %d tiles", max_tiles);
+  moe_tile_kernel<false><<<dim3((unsigned)((N + 63) / 64), (unsigned)max_tiles), dim3(256), 0, stream>>>(
+      (const bf16_t*)act, (int64_t)F, (const bf16_t*)down, (int64_t)F, order, offsets, tile_expert, tile_row, pair_weight, out, T, top, N, F);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ one wave per output element
+// act [P, F] in pair order (pair = token * top + choice): needs no sorting.
+template <typename TX>
+__global__ void __launch_bounds__(256)
+moe_gate_up_simple_kernel(const TX* __restrict__ x, int64_t ldx, const TX* __restrict__ gate_up, const int32_t* __restrict__ ids,
+                          TX* __restrict__ act, int64_t P, int top, int F, int K) {
+  const int lane = threadIdx.x & 63;
+  const int64_t at = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (at >= P * F) return;
+  const int64_t pair = at / F;
+  const int f = (int)(at - pair * F);
+  const TX* xr = x + (pair / top) * ldx;
+  const TX* gr = gate_up + ((int64_t)ids[pair] * 2 * F + f) * K;
+  const TX* ur = gr + (int64_t)F * K;
+  float sg = 0.f, su = 0.f;
+  for (int k = lane; k < K; k += 64) {
+    const float v = to_f32<TX>(xr[k]);
+    sg += v * to_f32<TX>(gr[k]);
+    su += v * to_f32<TX>(ur[k]);
+  }
+  sg = wave_sum(sg);
+  su = wave_sum(su);
+  if (lane == 0) act[at] = from_f32<TX>(sg / (1.f + expf(-sg)) * su);
+}
+
+template <typename TX>
+__global__ void __launch_bounds__(256)
+moe_down_simple_kernel(const TX* __restrict__ act, const TX* __restrict__ down, const int32_t* __restrict__ ids,
+                       const float* __restrict__ pair_weight, float* __restrict__ out, int64_t T, int top, int N, int F) {
+  const int lane = threadIdx.x & 63;
+  const int64_t at = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (at >= T * top * N) return;
+  const int64_t pair = at / N;
+  const int f = (int)(at - pair * N);
+  const TX* ar = act + pair * F;
+  const TX* dr = down + ((int64_t)ids[pair] * N + f) * F;
+  float s = 0.f;
+  for (int k = lane; k < F; k += 64) s += to_f32<TX>(ar[k]) * to_f32<TX>(dr[k]);
+  s = wave_sum(s);
+  const int64_t tok = pair / top, choice = pair - tok * top;
+  if (lane == 0) out[(choice * T + tok) * N + f] = s * pair_weight[pair];
+}
+
+extern "C" int me_moe_experts_simple(const void* x, int64_t ldx, int dtype, const void* gate_up, const void* down,
+                                     const int32_t* ids, const float* pair_weight, void* act, float* out, int64_t T, int top,
+                                     int N, int F, int K, hipStream_t stream) {
+  if (T == 0) return 0;
+  const int64_t P = T * top;
+  const int64_t g1 = (P * F + 3) / 4, g2 = (P * N + 3) / 4;
+  ME_CHECK(g1 < (1ll << 31) && g2 < (1ll << 31), "moe_experts_simple: too many outputs");
+  if (dtype == ME_F32) {
+    moe_gate_up_simple_kernel<float><<<dim3((unsigned)g1), dim3(256), 0, stream>>>((const float*)x, ldx, (const float*)gate_up, ids,
+                                                                                   (float*)act, P, top, F, K);
+    moe_down_simple_kernel<float><<<dim3((unsigned)g2), dim3(256), 0, stream>>>((const float*)act, (const float*)down, ids, pair_weight,
+                                                                                out, T, top, N, F);
+  } else {
+    moe_gate_up_simple_kernel<bf16_t><<<dim3((unsigned)g1), dim3(256), 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)gate_up, ids,
+                                                                                    (bf16_t*)act, P, top, F, K);
+    moe_down_simple_kernel<bf16_t><<<dim3((unsigned)g2), dim3(256), 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, ids,
+                                                                                 pair_weight, out, T, top, N, F);
+  }
+  ME_LAUNCH_CHECK();
+  return 0;
+}

@@ -32,3 +32,6 @@ class StepContext:
     # host copies, for parts that decide launches on the host
     q_lens: list = field(default_factory=list)
     starts: list = field(default_factory=list)
+    # what one layer call leaves for later calls of the same step, by name (values of this step's tokens that a
+    # later layer blends into its own); filled and read while the step runs, also while it is captured
+    shared: dict = field(default_factory=dict)

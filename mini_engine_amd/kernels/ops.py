@@ -77,6 +77,14 @@ _CORE_PROTOS = {
     "me_causal_conv": [P, L, I, P, P, P, L, P, P, I, P, L, I, I, I, P],
     "me_linear_recurrence": [P, L, P, L, P, L, I, P, L, P, P, P, P, P, L, P, P, P, L, I, I, I, I, I, I, I, I, I, I, P, P],
     "me_gated_rms_norm": [P, I, L, P, L, I, P, P, L, I, I, I, F, P],
+    "me_scaled_sum_norm": [P, I, I, P, P, P, P, P, F, P, P, P, P, P, I, L, I, F, P],
+    "me_softcap": [P, L, L, I, F, P],
+    "me_qkv_prepare": [P, L, P, P, P, F, I, I, F, I, P, P, P, P, P, L, I, L, I, I, I, I, I, I, P, P, L, P],
+    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P],
+    "me_moe_sort": [P, L, I, I, P, P, P, P, P],
+    "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, P],
+    "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, P],
+    "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
 }
@@ -694,6 +702,133 @@ class HipBackend:
                     weight.data_ptr(), out.data_ptr(), T, n, groups, GATED_NORMS[kind], float(eps), _stream())
         return out
 
+    # -- sublayers side by side, attention with biases and whole-projection norms ------------
+    def scaled_sum_norm(self, stream, terms, mult: float, w1, w2, eps: float, out_dtype: torch.dtype):
+        """stream' = stream + mult * sum_i scale_i * term_i, then y1 = w1 * stream' / rms(stream') and the same with w2,
+        one pass. stream: [T, n], float32 or the compute dtype (rows that start a stream); terms: up to four
+        (rows [T, n] in the compute dtype or float32 partial sums [P, T, n], scale float32 [n] or None); w1, w2: float32
+        [n] or None (w2 only with w1). Returns (stream' float32 [T, n], y1, y2) with y in out_dtype; without terms and
+        with a float32 stream, stream' is the stream itself."""
+        T, n = stream.shape
+        _check(stream.dim() == 2 and stream.is_contiguous(), "scaled_sum_norm: stream must be contiguous [T, n]")
+        _check(len(terms) <= 4, "scaled_sum_norm: up to four terms")
+        for w in (w1, w2):
+            _check(w is None or (w.dtype == torch.float32 and w.shape == (n,) and w.is_contiguous()), "scaled_sum_norm: norm weights float32 [n]")
+        _check(w2 is None or w1 is not None, "scaled_sum_norm: a second norm needs the first")
+        k = len(terms)
+        ptrs, dts, parts, strides, scales = (c_void_p * 4)(), (c_int * 4)(), (c_int * 4)(), (c_int64 * 4)(), (c_void_p * 4)()
+        for i, (t, sc) in enumerate(terms):
+            _check(t.is_contiguous() and t.shape[-2:] == (T, n) and (t.dim() == 2 or (t.dim() == 3 and t.dtype == torch.float32)),
+                   "scaled_sum_norm: a term is rows [T, n] or float32 partial sums [P, T, n]")
+            _check(sc is None or (sc.dtype == torch.float32 and sc.shape == (n,) and sc.is_contiguous()), "scaled_sum_norm: scales float32 [n]")
+            ptrs[i], dts[i], parts[i], strides[i] = t.data_ptr(), _code(t.dtype), (t.shape[0] if t.dim() == 3 else 1), T * n
+            scales[i] = None if sc is None else sc.data_ptr()
+        keep = k == 0 and stream.dtype == torch.float32
+        new = stream if keep else torch.empty((T, n), dtype=torch.float32, device=stream.device)
+        y1 = torch.empty((T, n), dtype=out_dtype, device=stream.device) if w1 is not None else None
+        y2 = torch.empty((T, n), dtype=out_dtype, device=stream.device) if w2 is not None else None
+        if keep and w1 is None:
+            return new, None, None
+        core().call("me_scaled_sum_norm", stream.data_ptr(), _code(stream.dtype), k, ptrs, dts, parts, strides, scales, float(mult),
+                    None if keep else new.data_ptr(), _ptr(w1), _ptr(w2), _ptr(y1), _ptr(y2), _code(out_dtype), T, n, float(eps), _stream())
+        return new, y1, y2
+
+    def softcap_(self, z: torch.Tensor, cap: float) -> torch.Tensor:
+        """z <- cap * tanh(z / cap) in place; float32 rows with unit inner stride."""
+        _check(z.dim() == 2 and z.dtype == torch.float32 and z.stride(1) == 1, "softcap: float32 rows")
+        core().call("me_softcap", z.data_ptr(), z.stride(0), z.shape[0], z.shape[1], float(cap), _stream())
+        return z
+
+    def qkv_prepare_store(self, rows, bias, q_weight, k_weight, eps: float, nq: int, nk: int, temperature, positions, slots,
+                          k_cache, v_cache, Hq: int, Hkv: int, D: int, page: int, vdim: int, mix: int = 0, lam=None,
+                          v_first=None) -> torch.Tensor:
+        """The step between a packed q/k/v product and attention, for projections with biases that are normed as a whole.
+        rows: float32 [T, (Hq + 2 Hkv) * D], the product's unrounded sums (heads in D slots each, slots beyond a head's
+        stored size zero); bias: float32 of that width or None; q_weight [Hq * D], k_weight [Hkv * D]: float32 weights
+        of an RMS norm over all of a token's query (key) slots at once, the mean taken over nq (nk) stored dimensions
+        (None: no norm); temperature: (coef, every) or None: the query at position p is multiplied by
+        1 + coef * ln(floor((p + 1) / every) + 1). mix 1: the first vdim slots of every value head are kept in v_first
+        (float32 [T, Hkv * vdim]); mix 2: v <- (1 - lam) v + lam v_first (lam: float32 tensor of one element). Keys and
+        values go to the pages at `slots` (K [pages, Hkv, page, D], V [pages, Hkv, D, page]; slots < 0 skipped).
+        Returns the queries [T, Hq * D] in the caches' dtype."""
+        T = rows.shape[0]
+        width = (Hq + 2 * Hkv) * D
+        _check(rows.dim() == 2 and rows.dtype == torch.float32 and rows.shape[1] >= width and rows.stride(1) == 1,
+               f"qkv_prepare_store: rows must be float32 [T, >= {width}]")
+        _check(bias is None or (bias.dtype == torch.float32 and bias.numel() >= width and bias.is_contiguous()), "qkv_prepare_store: bias float32")
+        _check((q_weight is None) == (k_weight is None), "qkv_prepare_store: both norm weights or neither")
+        if q_weight is not None:
+            _check(q_weight.dtype == torch.float32 and q_weight.shape == (Hq * D,) and q_weight.is_contiguous()
+                   and k_weight.dtype == torch.float32 and k_weight.shape == (Hkv * D,) and k_weight.is_contiguous(),
+                   "qkv_prepare_store: norm weights float32 [Hq * D] and [Hkv * D]")
+        _check(_is_i32(positions, T) and _is_i32(slots, T), "qkv_prepare_store: positions and slots int32 [T]")
+        _check(k_cache.dtype == v_cache.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+               and k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page),
+               "qkv_prepare_store: caches must be K [pages, Hkv, page, D] and V [pages, Hkv, D, page]")
+        if mix:
+            _check(v_first is not None and v_first.dtype == torch.float32 and v_first.shape == (T, Hkv * vdim) and v_first.stride(1) == 1
+                   and 1 <= vdim <= D, "qkv_prepare_store: v_first float32 [T, Hkv * vdim]")
+            _check(mix == 1 or (lam is not None and lam.dtype == torch.float32 and lam.numel() == 1), "qkv_prepare_store: lam float32 scalar")
+        coef, every = temperature if temperature else (0.0, 0)
+        q = torch.empty((T, Hq * D), dtype=k_cache.dtype, device=rows.device)
+        core().call("me_qkv_prepare", rows.data_ptr(), rows.stride(0), _ptr(bias), _ptr(q_weight), _ptr(k_weight), float(eps), int(nq),
+                    int(nk), float(coef), int(every), positions.data_ptr(), slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                    q.data_ptr(), q.stride(0), _code(k_cache.dtype), T, Hq, Hkv, D, page, int(vdim), int(mix),
+                    _ptr(lam) if mix == 2 else None, _ptr(v_first) if mix else None, v_first.stride(0) if mix else 0, _stream())
+        return q
+
+    # -- routed experts ------------------------------------------------------------------
+    def moe_route(self, x, router, top: int, group_count: int = 1, group_keep: int = 1):
+        """Which experts each token uses and with what weights. x: [T, n] rows; router: float32 [E, n]. Scores are the
+        softmax of router . x over all E experts, in float32. With group_count > 1 the experts form that many equal
+        groups of neighbours, a group scores as its best expert, and only experts of the group_keep best groups can be
+        chosen. The `top` largest scores are chosen (ties: the lower index); their weights are the scores divided by
+        their sum + 1e-20. Returns (ids int32 [T, top], weights float32 [T, top])."""
+        T, n = x.shape
+        E = router.shape[0]
+        _check(x.stride(1) == 1 and router.dtype == torch.float32 and router.shape == (E, n) and router.is_contiguous(),
+               "moe_route: rows [T, n], router float32 [E, n]")
+        ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
+        weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+        core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
+                    int(group_keep), ids.data_ptr(), weights.data_ptr(), _stream())
+        return ids, weights
+
+    def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False) -> torch.Tensor:
+        """Every token through its chosen gated experts: out[j, t] = weights[t, j] * W_down[e] (silu(W_gate[e] x_t) * (W_up[e] x_t)),
+        e = ids[t, j]: float32 [top, T, hidden], one partial sum per choice for a consumer that adds them. x: [T, K];
+        gate_up: [E, 2 F, K] (an expert's gate rows, then its up rows); down: [E, hidden, F]. bfloat16 with K and F in
+        whole steps of 8: the (token, choice) pairs are ordered by expert and cut into tiles of 64 rows, each tile one
+        workgroup of the matrix-core kernels; otherwise (float32, other sizes) one wave per output element."""
+        T, K = x.shape
+        top = ids.shape[1]
+        E, F2, _ = gate_up.shape
+        F, N = F2 // 2, down.shape[1]
+        _check(x.stride(1) == 1 and gate_up.is_contiguous() and down.is_contiguous() and gate_up.shape == (E, 2 * F, K)
+               and down.shape == (E, N, F) and gate_up.dtype == x.dtype and down.dtype == x.dtype, "routed_experts: operand shapes")
+        _check(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
+               and ids.shape == (T, top) and weights.shape == (T, top), "routed_experts: ids int32 [T, top], weights float32 [T, top]")
+        out = torch.empty((top, T, N), dtype=torch.float32, device=x.device)
+        Pn = T * top
+        act = torch.empty((Pn, F), dtype=x.dtype, device=x.device)
+        tiled = (x.dtype == torch.bfloat16 and K % 8 == 0 and F % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                 and not force_simple and Pn // 64 + min(E, Pn) <= 65535)
+        if not tiled:
+            core().call("me_moe_experts_simple", x.data_ptr(), x.stride(0), _code(x.dtype), gate_up.data_ptr(), down.data_ptr(),
+                        ids.data_ptr(), weights.data_ptr(), act.data_ptr(), out.data_ptr(), T, top, N, F, K, _stream())
+            return out
+        max_tiles = Pn // 64 + min(E, Pn)
+        meta = torch.empty((Pn + E + 1 + 2 * max_tiles,), dtype=torch.int32, device=x.device)
+        order, offsets = meta[:Pn], meta[Pn:Pn + E + 1]
+        tile_expert, tile_row = meta[Pn + E + 1:Pn + E + 1 + max_tiles], meta[Pn + E + 1 + max_tiles:]
+        core().call("me_moe_sort", ids.data_ptr(), Pn, E, max_tiles, order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
+                    tile_row.data_ptr(), _stream())
+        core().call("me_moe_gate_up", x.data_ptr(), x.stride(0), gate_up.data_ptr(), order.data_ptr(), offsets.data_ptr(),
+                    tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, _stream())
+        core().call("me_moe_down", act.data_ptr(), down.data_ptr(), order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
+                    tile_row.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, N, F, max_tiles, _stream())
+        return out
+
     # -- sampling ------------------------------------------------------------------------
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
         """Token ids int32 [S] from float32 logits [S, V]: argmax where temperature is 0, else
@@ -1257,3 +1392,8 @@ def head_gate(*a, **k): return backend().head_gate(*a, **k)
 def causal_conv(*a, **k): return backend().causal_conv(*a, **k)
 def linear_recurrence(*a, **k): return backend().linear_recurrence(*a, **k)
 def gated_rms_norm(*a, **k): return backend().gated_rms_norm(*a, **k)
+def scaled_sum_norm(*a, **k): return backend().scaled_sum_norm(*a, **k)
+def softcap_(*a, **k): return backend().softcap_(*a, **k)
+def qkv_prepare_store(*a, **k): return backend().qkv_prepare_store(*a, **k)
+def moe_route(*a, **k): return backend().moe_route(*a, **k)
+def routed_experts(*a, **k): return backend().routed_experts(*a, **k)

@@ -12,7 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..parts.base import CacheNeed, LayerCall, Part, Settled, StateNeed
-from ..parts.block import norm_of
+from ..parts.block import norm_of, settled
 
 
 @dataclass
@@ -115,6 +115,7 @@ class DecoderModel(Part):
         """Final norm of (h + residual), then the rows that want logits, then the head: float32
         [len(rows), vocab] (reference models/qwen3.py:91,116-117; layers/embed_head.py:19-23).
         `out`: where the head puts them (`parts.Head.forward(x, out)`)."""
+        h, residual = settled(h, residual)
         if isinstance(h, Settled):          # the last layer has added its output to the stream already: wanted rows first
             x, _ = self.final_norm.forward(ops.gather_rows(residual, rows), None)
             return self.head.forward(x, out=out)

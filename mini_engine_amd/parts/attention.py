@@ -11,6 +11,10 @@ from .base import CacheNeed, Mixer, ParamSpec, PositionEncoding, register_part
 from .linear import Linear
 
 
+def _half(shape, generator, device):
+    return 0.25 + 0.5 * torch.rand(shape, generator=generator, dtype=torch.float32, device=device)
+
+
 @register_part("mixer", "attention")
 class Attention(Mixer):
     """q, k, v from one packed product; optional per-head RMSNorm of q and k over the head
@@ -32,6 +36,14 @@ class Attention(Mixer):
     multiple of 16; the rotation's pairs half a head apart; rows in steps of 8), `finalize` builds it once: rows
     reordered within each head, zero rows and columns where a head is padded, the norm weights scaled so that a
     mean over the padded head equals the mean over the stored one.
+
+    A second family of options runs through a prologue kernel of its own (`ops.qkv_prepare_store`) on the unrounded
+    sums of the packed product: `qkv_bias` (q, k and v carry biases), `qk_norm_over="projection"` (q and k are each
+    normed as a whole, all heads at once, with weights of the projection's size; this needs no position encoding),
+    `q_temperature=(coef, every)` (the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)),
+    and `value_mix`: "first" keeps this layer's values of the step's tokens under `value_mix_key` in the step's shared
+    values; "blend" replaces its own by (1 - lambda) v + lambda v_first with a learned scalar lambda (`vmix`) before
+    they are cached. Layers that share a key have the same number of value dimensions.
     """
 
     takes_pending_norm = True      # x goes to the packed product and nowhere else
@@ -39,8 +51,21 @@ class Attention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, qk_norm_eps: float | None = None, position: PositionEncoding | None = None,
                  window: int | None = None, own_kv: bool = True, value_dim: int | None = None,
-                 chunk: int | None = None, head_gate: bool = False):
+                 chunk: int | None = None, head_gate: bool = False, qkv_bias: bool = False, qk_norm_over: str = "head",
+                 q_temperature: tuple | None = None, value_mix: str | None = None, value_mix_key: str = "v_first"):
         super().__init__()
+        if qk_norm_over not in ("head", "projection") or value_mix not in (None, "first", "blend"):
+            raise ValueError("qk_norm_over is 'head' or 'projection', value_mix None, 'first' or 'blend'")
+        self.qkv_bias_on = bool(qkv_bias)
+        self.norm_over = qk_norm_over
+        self.q_temperature = None if q_temperature is None else (float(q_temperature[0]), int(q_temperature[1]))
+        if self.q_temperature is not None and self.q_temperature[1] < 1:
+            raise ValueError("the query temperature's period must be positive")
+        self.value_mix, self.value_mix_key = value_mix, value_mix_key
+        self.prologue = bool(qkv_bias or qk_norm_over == "projection" or q_temperature is not None or value_mix)
+        if self.prologue and (position is not None or not own_kv or head_gate or (qk_norm_eps is not None and qk_norm_over == "head")):
+            raise ValueError("biases, whole-projection norms, query temperatures and value mixing come without a position "
+                             "encoding, head gates or per-head norms, on keys and values of the layer's own")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         self.hidden_size = hidden_size
@@ -80,9 +105,14 @@ class Attention(Mixer):
         self.gate_at = self.q_size + (2 * self.kv_size if own_kv else 0)      # first gate column of the kernels' rows
         self._laid_out = False
         if qk_norm_eps is not None:
-            self.add_param("q_norm_weight", ParamSpec((self.stored_dim,), init="norm", dtype="float32"))
+            whole = qk_norm_over == "projection"
+            self.add_param("q_norm_weight", ParamSpec((stored_q if whole else self.stored_dim,), init="norm", dtype="float32"))
             if own_kv:
-                self.add_param("k_norm_weight", ParamSpec((self.stored_dim,), init="norm", dtype="float32"))
+                self.add_param("k_norm_weight", ParamSpec((stored_k if whole else self.stored_dim,), init="norm", dtype="float32"))
+        if qkv_bias:
+            self.add_param("qkv_bias", ParamSpec((stored_q + stored_k + stored_v,), init="matrix", dtype="float32"))
+        if value_mix == "blend":
+            self.add_param("vmix", ParamSpec((), init=_half, dtype="float32"))
         self.norm_eps = qk_norm_eps
         if position is not None:
             self.add_child("position", position)
@@ -126,7 +156,17 @@ class Attention(Mixer):
         self.qkv.weight = torch.cat(parts, 0).contiguous()
         o = self.o.weight.view(-1, H, nv)
         self.o.weight = torch.cat((o, o.new_zeros(o.shape[0], H, D - nv)), 2).reshape(-1, H * D).contiguous()
-        if self.norm_eps is not None:
+        if self.qkv_bias_on:
+            b = self.qkv_bias
+            wide = lambda block, count, size, pick: torch.cat((block.view(count, size), block.new_zeros(count, 1)), 1)[:, pick.to(block.device)].reshape(-1)
+            self.qkv_bias = torch.cat((wide(b[:stored_q], H, n, take), wide(b[stored_q:stored_q + stored_k], G, n, take),
+                                       wide(b[stored_q + stored_k:], G, nv, keep))).contiguous()
+        if self.norm_eps is not None and self.norm_over == "projection":
+            # the kernel divides the sum of squares by the stored count itself: the weights only move to their slots
+            for name, count in (("q_norm_weight", H), ("k_norm_weight", G)):
+                wn = getattr(self, name)
+                setattr(self, name, torch.cat((wn.view(count, n), wn.new_zeros(count, 1)), 1)[:, take.to(wn.device)].reshape(-1).contiguous())
+        elif self.norm_eps is not None:
             # mean over D slots instead of n stored dimensions: eps and the weights take the ratio
             self.qk_norm_eps = self.norm_eps * n / D
             fix = math.sqrt(n / D)
@@ -136,7 +176,36 @@ class Attention(Mixer):
                 setattr(self, name, wide[take.to(wn.device)].contiguous())
         self._laid_out = True
 
+    def _forward_with_prologue(self, x, step, cache):
+        """Bias, whole-projection norm, temperature and value mixing on the product's float32 sums, then attention."""
+        Hq, Hkv, D, nv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        grp = step.groups[cache.group]
+        rows = self.qkv.forward(x, out_dtype=torch.float32)
+        mix, v_first = 0, None
+        if self.value_mix is not None:
+            if self.value_mix == "first":
+                mix, v_first = 1, torch.empty((rows.shape[0], Hkv * nv), dtype=torch.float32, device=rows.device)
+                step.shared[self.value_mix_key] = v_first
+            else:
+                mix, v_first = 2, step.shared.get(self.value_mix_key)
+                if v_first is None or v_first.shape != (rows.shape[0], Hkv * nv):
+                    raise RuntimeError(f"value mixing: no layer before this one has left {Hkv * nv} value dimensions "
+                                       f"per token under {self.value_mix_key!r}")
+        normed = self.norm_eps is not None
+        q = ops.qkv_prepare_store(rows, self.qkv_bias if self.qkv_bias_on else None, self.q_norm_weight if normed else None,
+                                  self.k_norm_weight if normed else None, self.norm_eps or 0.0, Hq * self.stored_dim,
+                                  Hkv * self.stored_dim, self.q_temperature, step.positions, grp.slot_mapping, cache.k, cache.v,
+                                  Hq, Hkv, D, cache.page_size, nv, mix, self.vmix if mix == 2 else None, v_first)
+        o = ops.paged_attention(q, cache.k, cache.v, cache.page_size, grp.block_tables, step.context_lens,
+                                step.seq_of_token, step.positions, step.prefill_cu, step.num_decodes,
+                                step.max_decode_context, self.scale, self.window, Hq, Hkv, D,
+                                max_prefill_context=step.max_prefill_context,
+                                even_contexts=step.decode_contexts_even, chunk=self.chunk)
+        return self.o.forward(o, allow_partials=True)
+
     def forward(self, x, step, cache, state):
+        if self.prologue:
+            return self._forward_with_prologue(x, step, cache)
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         grp = step.groups[cache.group]
         packed = self.qkv.forward(x)

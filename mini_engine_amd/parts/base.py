@@ -234,6 +234,22 @@ class Settled:
         self.rounded = rounded
 
 
+class ScaledSum:
+    """What a layer returns in place of its output when several sublayer outputs still have to be added to the
+    residual stream, each under a scale of its own: stream += mult * sum_i scale_i * term_i. `terms`: pairs of (rows
+    [T, n] in the compute dtype or float32 partial sums [P, T, n], float32 scale [n] or None). Whoever runs next forms
+    the sum, a block of the same kind together with its own norms in one pass (`ops.scaled_sum_norm`); anyone else
+    calls `settle`."""
+
+    def __init__(self, terms: list, mult: float):
+        self.terms, self.mult = list(terms), float(mult)
+
+    def settle(self, stream: torch.Tensor) -> torch.Tensor:
+        """The new stream, float32 [T, n]."""
+        from ..kernels import ops
+        return ops.scaled_sum_norm(stream, self.terms, self.mult, None, None, 0.0, torch.float32)[0]
+
+
 class PositionEncoding(Part):
     """Something applied to queries and keys as a function of token positions."""
 
@@ -268,6 +284,8 @@ class Mixer(Part):
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """[T, hidden] -> [T, hidden], or float32 partial sums [P, T, hidden], or a tuple of such tensors whose sum is
+        the output (a routed part beside one that every token passes)."""
         raise NotImplementedError
 
 

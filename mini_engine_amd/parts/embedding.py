@@ -22,11 +22,13 @@ class LMHead(Head):
     """logits = x . W^T in float32. When tied, W is the embedding matrix itself: the same
     tensor, not a copy (reference models/qwen3.py:107-109)."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, softcap: float | None = None):
+        """`softcap`: the logits are bent into (-softcap, softcap): z <- softcap * tanh(z / softcap)."""
         super().__init__()
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied_to = tied_to
+        self.softcap = None if softcap is None else float(softcap)
         if tied_to is None:
             self.add_param("weight", ParamSpec((vocab_size, hidden_size), init="matrix", dtype="compute"))
 
@@ -36,4 +38,5 @@ class LMHead(Head):
     def forward(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """`out`: a float32 [rows, vocab] tensor to write the logits into (a step with a fixed layout
         keeps one)."""
-        return ops.linear(x, self.matrix(), torch.float32, out=out)
+        z = ops.linear(x, self.matrix(), torch.float32, out=out)
+        return z if self.softcap is None else ops.softcap_(z, self.softcap)

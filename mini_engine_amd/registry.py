@@ -49,4 +49,4 @@ def build_model(model_config, checkpoint_names=None):
 
 
 def _load_builtin() -> None:
-    from .models import qwen3, sigosun  # noqa: F401  (they register themselves)
+    from .models import negosun, qwen3, sigosun  # noqa: F401  (they register themselves)

@@ -73,8 +73,7 @@ def check_checkpoint(model, index: dict) -> None:
         if spec is None:
             raise WeightError(f"weight source given for {pname!r}, which is not a parameter of the model")
         for src in sources:
-            rows = spec.shape[0] if src.rows is None else src.rows
-            expect = (rows,) + tuple(spec.shape[1:])
+            expect = tuple(spec.shape) if src.rows is None else (src.rows,) + tuple(spec.shape[1:])      # a scalar has no rows
             if src.name not in index:
                 missing.append(f"{src.name} {list(expect)}")
                 continue

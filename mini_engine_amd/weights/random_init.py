@@ -22,8 +22,8 @@ def _checkpoint_tensor_specs(model) -> list:
     for pname, sources in model.weight_sources.items():
         spec = specs[pname]
         for src in sources:
-            rows = spec.shape[0] if src.rows is None else src.rows
-            out[src.name] = ((rows,) + tuple(spec.shape[1:]), spec.init, spec.dtype)
+            shape = tuple(spec.shape) if src.rows is None else (src.rows,) + tuple(spec.shape[1:])
+            out[src.name] = (shape, spec.init, spec.dtype)
     return sorted((n, s, k, d) for n, (s, k, d) in out.items())
 
 

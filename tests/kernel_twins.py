@@ -253,6 +253,89 @@ def gated_rms_norm(y, gate, weight, eps, groups, kind, out_dtype):
     return r.to(out_dtype)
 
 
+def scaled_sum_norm(stream, terms, mult, w1, w2, eps, out_dtype):
+    """stream + mult * sum_i scale_i * term_i in float32, then up to two RMS norms of it."""
+    new = stream.float()
+    if terms:
+        add = torch.zeros_like(new)
+        for t, sc in terms:
+            v = t.float().sum(0) if t.dim() == 3 else t.float()
+            add = add + (v if sc is None else sc * v)
+        new = new + mult * add
+    elif stream.dtype == torch.float32:
+        new = stream
+    u = new * torch.rsqrt(new.pow(2).mean(-1, keepdim=True) + eps)
+    return new, (None if w1 is None else (u * w1).to(out_dtype)), (None if w2 is None else (u * w2).to(out_dtype))
+
+
+def softcap_(z, cap):
+    z.copy_(cap * torch.tanh(z / cap))
+    return z
+
+
+def qkv_prepare_store(rows, bias, q_weight, k_weight, eps, nq, nk, temperature, positions, slots, k_cache, v_cache,
+                      Hq, Hkv, D, page, vdim, mix=0, lam=None, v_first=None):
+    T = rows.shape[0]
+    wq, wk = Hq * D, Hkv * D
+    r = rows[:, :wq + 2 * wk].float()
+    if bias is not None:
+        r = r + bias[:wq + 2 * wk]
+    q, k, v = r[:, :wq], r[:, wq:wq + wk], r[:, wq + wk:].clone()
+    if q_weight is not None:
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) / nq + eps) * q_weight
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) / nk + eps) * k_weight
+    if temperature:
+        coef, every = temperature
+        steps = torch.div(positions[:T].long() + 1, every, rounding_mode="floor").float()
+        q = q * (1.0 + coef * torch.log(steps + 1.0))[:, None]
+    if mix:
+        real = v.view(T, Hkv, D)[:, :, :vdim]
+        if mix == 1:
+            v_first.copy_(real.reshape(T, Hkv * vdim))
+        else:
+            real.copy_((1.0 - lam.float()) * real + lam.float() * v_first.view(T, Hkv, vdim))
+    dt = k_cache.dtype
+    write_pages(k.reshape(T, Hkv, D).to(dt), v.reshape(T, Hkv, D).to(dt), slots[:T], k_cache, v_cache, page)
+    return q.to(dt).contiguous()
+
+
+def moe_route(x, router, top, group_count=1, group_keep=1):
+    z = x.float() @ router.float().t()
+    s = torch.softmax(z, dim=-1)
+    T, E = s.shape
+    m = s.clone()
+    if group_count > 1 and group_keep < group_count:
+        per = E // group_count
+        gs = s.view(T, group_count, per).amax(-1)
+        kept = torch.zeros((T, group_count), dtype=torch.bool, device=x.device)
+        for _ in range(group_keep):
+            best = torch.where(kept, torch.full_like(gs, -2.0), gs).argmax(-1)      # ties: the lower index
+            kept[torch.arange(T), best] = True
+        m = torch.where(kept.repeat_interleave(per, 1), m, torch.full_like(m, -1.0))
+    ids = torch.empty((T, top), dtype=torch.int64, device=x.device)
+    for j in range(top):
+        best = m.argmax(-1)
+        ids[:, j] = best
+        m[torch.arange(T), best] = -2.0
+    w = torch.gather(s, 1, ids)
+    return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20)).float()
+
+
+def routed_experts(x, ids, weights, gate_up, down, force_simple=False):
+    T, K = x.shape
+    top = ids.shape[1]
+    F = gate_up.shape[1] // 2
+    out = torch.zeros((top, T, down.shape[1]), dtype=torch.float32, device=x.device)
+    xf = x.float()
+    for j in range(top):
+        for e in ids[:, j].unique().tolist():
+            rows = (ids[:, j] == e).nonzero().flatten()
+            gu = xf[rows] @ gate_up[e].float().t()
+            act = (gu[:, :F] * torch.sigmoid(gu[:, :F]) * gu[:, F:]).to(x.dtype).float()
+            out[j, rows] = (act @ down[e].float().t()) * weights[rows, j][:, None]
+    return out
+
+
 def _fmix32(h):
     m = 0xFFFFFFFF
     h = h & m
@@ -326,3 +409,8 @@ class PlainBackend:
     causal_conv = staticmethod(causal_conv)
     linear_recurrence = staticmethod(linear_recurrence)
     gated_rms_norm = staticmethod(gated_rms_norm)
+    scaled_sum_norm = staticmethod(scaled_sum_norm)
+    softcap_ = staticmethod(softcap_)
+    qkv_prepare_store = staticmethod(qkv_prepare_store)
+    moe_route = staticmethod(moe_route)
+    routed_experts = staticmethod(routed_experts)
