@@ -37,7 +37,7 @@ import time
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-from mini_engine_amd.config.sizes import SIZES, model_config, sigosun_config   # noqa: E402  (the named layer sizes)
+from mini_engine_amd.config.sizes import SIZES, model_config, named_config   # noqa: E402  (the named layer sizes)
 
 
 def log(msg: str) -> None:
@@ -67,17 +67,28 @@ def _matrix_params(model) -> tuple:
     runs = _used_per_call(model)
     tied = getattr(model.head, "tied_to", None) is model.embedding
     per_token = head = 0
-    for name, _, _, spec in model.named_specs():
+    for name, part, local, spec in model.named_specs():
         if len(spec.shape) < 2:
             continue
         n = 1
         for d in spec.shape:
             n *= int(d)
+        n *= _routed_share(part, local, 1)          # a token passes `top` of a routed part's experts
         if name.startswith("layers."):
             per_token += n * runs.get(int(name.split(".")[1]), 0)
         elif name.startswith("head.") or (tied and name.startswith("embedding.")):
             head += n
     return per_token, head
+
+
+def _routed_share(part, local: str, tokens: int) -> float:
+    """The share of a parameter that a step of `tokens` tokens reads: 1, or for the packed expert matrices of a routed
+    feed-forward the expected share of experts that some token chooses (choices taken as uniform over the experts; one
+    token: top / experts)."""
+    experts, top = getattr(part, "num_experts", None), getattr(part, "top", None)
+    if not experts or local not in ("gate_up", "down"):
+        return 1.0
+    return 1.0 - (1.0 - top / experts) ** tokens
 
 
 def cache_bytes_per_token(model, page: int, dtype) -> list:
@@ -92,7 +103,7 @@ def decode_bytes(model, item: int, contexts: list, page: int, dtype) -> int:
     head's matrix as well: a step gathers a row per request from it), and what the cache holds of the live requests
     (a windowed group at most its window)."""
     tied = getattr(model.head, "tied_to", None) is model.embedding
-    weights = sum(_spec_bytes(spec, item) for name, _, _, spec in model.named_specs()
+    weights = sum(_spec_bytes(spec, item) * _routed_share(part, local, len(contexts)) for name, part, local, spec in model.named_specs()
                   if tied or not name.startswith("embedding."))
     kv = 0.0
     for per_token, window in cache_bytes_per_token(model, page, dtype):
@@ -324,13 +335,13 @@ def resolve_model(args, size: str, layers, tmp: str) -> tuple:
         if stored:
             return cfg, full, label, size, None, "the folder's checkpoint"
         return cfg, full, label, size, args.seed, "drawn on the device"
-    design = size.startswith("sigosun:")
-    cfg, full = sigosun_config(size.split(":")[1], layers) if design else model_config(size, layers)
+    design = size.split(":")[0] if ":" in size else None
+    cfg, full = named_config(size, layers)
     skeleton = build_model(cfg)                              # declared parameters only, no tensors
     params = sum(_spec_bytes(spec, 1) for _, _, _, spec in skeleton.named_specs())
     on_device = args.weights == "device" or (args.weights == "auto" and params > 2e9)
     folder, random_weights = folder_for(cfg, args.seed, os.path.join(tmp, size.replace(":", "_")), on_device)
-    label = f"Sigosun at the Qwen3-{size.split(':')[1]} layer sizes" if design else f"Qwen3-{size} sizes"
+    label = f"{design.capitalize()} at the Qwen3-{size.split(':')[1]} layer sizes" if design else f"Qwen3-{size} sizes"
     return cfg, full, label, folder, random_weights, "drawn on the device" if on_device else "written folder"
 
 
@@ -456,7 +467,7 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
-    ap.add_argument("--design", default=None, choices=["sigosun"],
+    ap.add_argument("--design", default=None, choices=["sigosun", "negosun"],
                     help="instead of the default workload: prefill and decode throughput of this design at the layer sizes "
                          "named by --design-sizes (random weights), each beside Qwen3 at the same width, depth and vocabulary")
     ap.add_argument("--design-sizes", default="0.6b,8b")

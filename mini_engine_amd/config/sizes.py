@@ -3,7 +3,7 @@ with random weights (no model folder at hand). The figures are those of the publ
 files; a model folder's own config.json always wins where there is one."""
 from __future__ import annotations
 
-from .model_config import Qwen3Config, SigosunConfig
+from .model_config import NegosunConfig, Qwen3Config, SigosunConfig
 
 SIZES = {
     # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
@@ -59,10 +59,29 @@ def sigosun_config(size: str, layers: int | None = None):
                                     "max_position_embeddings": 40960}), L
 
 
+def negosun_config(size: str, layers: int | None = None):
+    """(a Negosun configuration whose layers resemble that size's: the same width, vocabulary and attention heads, with
+    `layers` layers or as many as the size has; that count). Every layer mixes its values with the first layer's and has a
+    query temperature that steps every 1,024 positions. The feed-forward has 32 experts of an eighth of the size's
+    feed-forward width in four groups of which two are kept, four experts per token, and a shared expert of half that
+    width: a token passes as many feed-forward weights as in the dense model of that size."""
+    L, h, Hq, Hkv, D, I, V, _ = SIZES[size]
+    n = layers or L
+    ff = max(8, I // 8)
+    layer = {"type": "attention",
+             "mixer": {"heads": Hq, "kv_heads": Hkv, "dim": D, "vdim": D, "scale": D ** -0.5, "v_mix": True, "q_temp": {"coef": 0.1, "every": 1024}},
+             "mlp": {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": max(8, I // 2)},
+                     "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}}}}
+    return NegosunConfig.from_dict({"architecture": "Negosun", "vocab": V, "width": h, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+                                    "logit_softcap": 30.0, "layers": [layer] * n, "max_position_embeddings": 40960}), L
+
+
 def named_config(name: str, layers: int | None = None):
     """(configuration, full layer count) of a name the command lines take for random weights: a Qwen3 size
-    ("0.6b"), or "sigosun:<size>" for the Sigosun design at that size's layer sizes."""
+    ("0.6b"), or "sigosun:<size>" / "negosun:<size>" for those designs at that size's layer sizes."""
     design, _, size = name.rpartition(":")
-    if size not in SIZES or design not in ("", "qwen3", "sigosun"):
-        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:'")
+    if size not in SIZES or design not in ("", "qwen3", "sigosun", "negosun"):
+        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:' or 'negosun:'")
+    if design == "negosun":
+        return negosun_config(size, layers)
     return sigosun_config(size, layers) if design == "sigosun" else model_config(size, layers)
