@@ -37,19 +37,15 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// One workgroup of 4 waves per `tokens_per_group` tokens (their rows wait in LDS); a wave takes every fourth expert's
-// dot products, then every fourth token's selection. LDS: rows, then per token E scores, E working copies, and the
-// group scores.
+// Router logits: a workgroup of 4 waves takes `tokens_per_group` tokens (their rows wait in LDS) and `experts_per_group`
+// experts, a wave every fourth of them; a lane walks K in steps of 64 and the wave adds up. float32 [T, E] out.
 template <typename TX>
 __global__ void __launch_bounds__(256)
-moe_route_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t T, int n, int E, int top,
-                 int group_count, int group_keep, int tokens_per_group, int32_t* __restrict__ ids, float* __restrict__ weights) {
+moe_logits_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t T, int n, int E,
+                  int tokens_per_group, int experts_per_group, float* __restrict__ logits) {
   extern __shared__ __align__(16) unsigned char route_lds[];
   const int TT = tokens_per_group;
   TX* xs = reinterpret_cast<TX*>(route_lds);
-  float* score = reinterpret_cast<float*>(route_lds + (((size_t)TT * n * sizeof(TX) + 15) & ~(size_t)15));
-  float* work = score + (size_t)TT * E;
-  float* gscore = work + (size_t)TT * E;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t t0 = (int64_t)blockIdx.x * TT;
   const int live = (int)min((int64_t)TT, T - t0);
@@ -58,81 +54,104 @@ moe_route_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict_
     xs[i] = tt < live ? x[(t0 + tt) * ldx + k] : from_f32<TX>(0.f);
   }
   __syncthreads();
-  for (int e = wave; e < E; e += 4) {
+  const int e0 = blockIdx.y * experts_per_group, e1 = min(E, e0 + experts_per_group);
+  const bool vec = (n & 3) == 0;           // rows in whole groups of 4: a lane takes 4 neighbours at a time
+  for (int e = e0 + wave; e < e1; e += 4) {
     float acc[8];
 #pragma unroll
     for (int tt = 0; tt < 8; ++tt) acc[tt] = 0.f;
     const float* we = w + (int64_t)e * n;
-    for (int k = lane; k < n; k += 64) {
-      const float wv = we[k];
+    if (vec) {
+#pragma unroll 4
+      for (int k = lane * 4; k < n; k += 256) {
+        const float4 wv = *reinterpret_cast<const float4*>(we + k);
 #pragma unroll
-      for (int tt = 0; tt < 8; ++tt)
-        if (tt < TT) acc[tt] += wv * to_f32<TX>(xs[tt * n + k]);
+        for (int tt = 0; tt < 8; ++tt)
+          if (tt < TT) {
+            const TX* xr = xs + tt * n + k;
+            acc[tt] += wv.x * to_f32<TX>(xr[0]) + wv.y * to_f32<TX>(xr[1]) + wv.z * to_f32<TX>(xr[2]) + wv.w * to_f32<TX>(xr[3]);
+          }
+      }
+    } else {
+      for (int k = lane; k < n; k += 64) {
+        const float wv = we[k];
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt)
+          if (tt < TT) acc[tt] += wv * to_f32<TX>(xs[tt * n + k]);
+      }
     }
 #pragma unroll
     for (int tt = 0; tt < 8; ++tt)
       if (tt < TT) {
         const float s = wave_sum(acc[tt]);
-        if (lane == 0) score[tt * E + e] = s;
+        if (lane == 0 && tt < live) logits[(t0 + tt) * E + e] = s;
       }
-  }
-  __syncthreads();
-  const int per = E / group_count;
-  for (int tt = wave; tt < live; tt += 4) {
-    float* s = score + tt * E;
-    float* m = work + tt * E;
-    float* gs = gscore + tt * group_count;
-    float hi = -INFINITY;
-    for (int e = lane; e < E; e += 64) hi = fmaxf(hi, s[e]);
-    hi = wave_max(hi);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) { const float p = expf(s[e] - hi); s[e] = p; sum += p; }
-    sum = wave_sum(sum);
-    for (int e = lane; e < E; e += 64) { s[e] = s[e] / sum; m[e] = s[e]; }
-    wave_settle();
-    if (group_count > 1 && group_keep < group_count) {
-      for (int g = lane; g < group_count; g += 64) {
-        float best = -1.f;
-        for (int j = 0; j < per; ++j) best = fmaxf(best, s[g * per + j]);
-        gs[g] = best;
-      }
-      wave_settle();
-      // the best groups one after the other; a kept group's score drops to -2, the others' experts leave the race
-      for (int kept = 0; kept < group_keep; ++kept) {
-        float bv = -3.f; int bi = 0x7fffffff;
-        for (int g = lane; g < group_count; g += 64)
-          if (gs[g] > bv) { bv = gs[g]; bi = g; }
-        wave_argmax(bv, bi);
-        if (bi >= group_count) bi = 0;          // scores that are no numbers: still a valid index
-        if (lane == 0) gs[bi] = -2.f;
-        wave_settle();
-      }
-      for (int e = lane; e < E; e += 64)
-        if (gs[e / per] != -2.f) m[e] = -1.f;
-      wave_settle();
-    }
-    float total = 0.f;
-    int mine = -1;           // lane j keeps the j-th choice (top <= 64)
-    for (int j = 0; j < top; ++j) {
-      float bv = -3.f; int bi = 0x7fffffff;
-      for (int e = lane; e < E; e += 64)
-        if (m[e] > bv) { bv = m[e]; bi = e; }
-      wave_argmax(bv, bi);
-      if (bi >= E) bi = 0;
-      if (lane == 0) m[bi] = -2.f;
-      wave_settle();
-      if (lane == j) mine = bi;
-      total += s[bi];
-    }
-    if (lane < top) {
-      ids[(t0 + tt) * top + lane] = mine;
-      weights[(t0 + tt) * top + lane] = s[mine] / (total + 1e-20f);
-    }
   }
 }
 
+// The choice: a wave per token (4 tokens a workgroup). LDS per token: E scores, E working copies, the group scores.
+__global__ void __launch_bounds__(256)
+moe_select_kernel(const float* __restrict__ logits, int64_t T, int E, int top, int group_count, int group_keep,
+                  int32_t* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ __align__(16) unsigned char route_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float* s = reinterpret_cast<float*>(route_lds) + (size_t)wave * (2 * E + group_count);
+  float* m = s + E;
+  float* gs = m + E;
+  const int per = E / group_count;
+  float hi = -INFINITY;
+  for (int e = lane; e < E; e += 64) { s[e] = logits[t * E + e]; hi = fmaxf(hi, s[e]); }
+  hi = wave_max(hi);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) { const float p = expf(s[e] - hi); s[e] = p; sum += p; }
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += 64) { s[e] = s[e] / sum; m[e] = s[e]; }
+  wave_settle();
+  if (group_count > 1 && group_keep < group_count) {
+    for (int g = lane; g < group_count; g += 64) {
+      float best = -1.f;
+      for (int j = 0; j < per; ++j) best = fmaxf(best, s[g * per + j]);
+      gs[g] = best;
+    }
+    wave_settle();
+    // the best groups one after the other; a kept group's score drops to -2, the others' experts leave the race
+    for (int kept = 0; kept < group_keep; ++kept) {
+      float bv = -3.f; int bi = 0x7fffffff;
+      for (int g = lane; g < group_count; g += 64)
+        if (gs[g] > bv) { bv = gs[g]; bi = g; }
+      wave_argmax(bv, bi);
+      if (bi >= group_count) bi = 0;          // scores that are no numbers: still a valid index
+      if (lane == 0) gs[bi] = -2.f;
+      wave_settle();
+    }
+    for (int e = lane; e < E; e += 64)
+      if (gs[e / per] != -2.f) m[e] = -1.f;
+    wave_settle();
+  }
+  float total = 0.f;
+  int mine = 0;              // lane j keeps the j-th choice (top <= 64)
+  for (int j = 0; j < top; ++j) {
+    float bv = -3.f; int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64)
+      if (m[e] > bv) { bv = m[e]; bi = e; }
+    wave_argmax(bv, bi);
+    if (bi >= E) bi = 0;
+    if (lane == 0) m[bi] = -2.f;
+    wave_settle();
+    if (lane == j) mine = bi;
+    total += s[bi];
+  }
+  if (lane < top) {
+    ids[t * top + lane] = mine;
+    weights[t * top + lane] = s[mine] / (total + 1e-20f);
+  }
+}
+
+// logits: float32 [T, E] working memory.
 extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* w, int64_t T, int n, int E, int top,
-                            int group_count, int group_keep, int32_t* ids, float* weights, hipStream_t stream) {
+                            int group_count, int group_keep, float* logits, int32_t* ids, float* weights, hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && top >= 1 && top <= 64 && top <= E, "moe_route: %d experts, top %d", E, top);
   ME_CHECK(group_count >= 1 && E % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
@@ -140,26 +159,30 @@ extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* 
   ME_CHECK(group_keep * (E / group_count) >= top, "moe_route: the kept groups hold fewer than top experts");
   const size_t es = dtype == ME_F32 ? 4 : 2;
   int TT = 8;
-  while (TT > 1 && (size_t)TT * n * es > 32 * 1024) TT >>= 1;
-  const size_t lds = (((size_t)TT * n * es + 15) & ~(size_t)15) + (size_t)TT * (2 * E + group_count) * 4;
-  ME_CHECK(lds <= 64 * 1024, "moe_route: width %d with %d experts does not fit a workgroup's memory", n, E);
+  while (TT > 1 && ((size_t)TT * n * es > 32 * 1024 || TT / 2 >= T)) TT >>= 1;       // as many as fit, and no more than there are
+  ME_CHECK((size_t)TT * n * es <= 64 * 1024, "moe_route: a row of %d does not fit a workgroup's memory", n);
   const int64_t groups = (T + TT - 1) / TT;
-  ME_CHECK(groups < (1ll << 31), "moe_route: too many tokens");
+  ME_CHECK(groups < (1ll << 31) && (T + 3) / 4 < (1ll << 31), "moe_route: too many tokens");
+  // few tokens: the experts spread over as many workgroups as possible; many: a workgroup keeps its rows for 32 experts
+  const int per_group = groups <= 64 ? 4 : 32;
+  const dim3 grid((unsigned)groups, (unsigned)((E + per_group - 1) / per_group));
   if (dtype == ME_F32)
-    moe_route_kernel<float><<<dim3((unsigned)groups), dim3(256), lds, stream>>>((const float*)x, ldx, w, T, n, E, top, group_count,
-                                                                                group_keep, TT, ids, weights);
+    moe_logits_kernel<float><<<grid, dim3(256), (size_t)TT * n * es, stream>>>((const float*)x, ldx, w, T, n, E, TT, per_group, logits);
   else
-    moe_route_kernel<bf16_t><<<dim3((unsigned)groups), dim3(256), lds, stream>>>((const bf16_t*)x, ldx, w, T, n, E, top, group_count,
-                                                                                 group_keep, TT, ids, weights);
+    moe_logits_kernel<bf16_t><<<grid, dim3(256), (size_t)TT * n * es, stream>>>((const bf16_t*)x, ldx, w, T, n, E, TT, per_group, logits);
+  ME_LAUNCH_CHECK();
+  const size_t lds = (size_t)4 * (2 * E + group_count) * 4;
+  ME_CHECK(lds <= 64 * 1024, "moe_route: %d experts do not fit a workgroup's memory", E);
+  moe_select_kernel<<<dim3((unsigned)((T + 3) / 4)), dim3(256), lds, stream>>>(logits, T, E, top, group_count, group_keep, ids, weights);
   ME_LAUNCH_CHECK();
   return 0;
 }
 
 // ------------------------------------------------------------------ pairs by expert
 // One workgroup. order[p']: the pair at sorted place p'; offsets[e]: where expert e's pairs begin; tile_expert / tile_row:
-// expert and first sorted place of every tile of up to 64 pairs (expert -1: a tile nobody needs).
+// expert and first sorted place of every tile of up to `tile_rows` pairs (expert -1: a tile nobody needs).
 __global__ void __launch_bounds__(1024)
-moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, int32_t* __restrict__ order,
+moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, int tile_rows, int32_t* __restrict__ order,
                 int32_t* __restrict__ offsets, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row) {
   __shared__ int count[MOE_MAX_EXPERTS], begin[MOE_MAX_EXPERTS + 1], tile_at[MOE_MAX_EXPERTS + 1], cursor[MOE_MAX_EXPERTS];
   for (int e = threadIdx.x; e < E; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
@@ -171,7 +194,7 @@ moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, in
     for (int e = 0; e < E; ++e) {
       begin[e] = at; tile_at[e] = tiles;
       at += count[e];
-      tiles += (count[e] + MOE_TM - 1) / MOE_TM;
+      tiles += (count[e] + tile_rows - 1) / tile_rows;
     }
     begin[E] = at; tile_at[E] = tiles;
   }
@@ -184,17 +207,18 @@ moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, in
   for (int e = threadIdx.x; e < E; e += blockDim.x)
     for (int i = tile_at[e]; i < tile_at[e + 1] && i < max_tiles; ++i) {
       tile_expert[i] = e;
-      tile_row[i] = begin[e] + (i - tile_at[e]) * MOE_TM;
+      tile_row[i] = begin[e] + (i - tile_at[e]) * tile_rows;
     }
   for (int i = tile_at[E] + threadIdx.x; i < max_tiles; i += blockDim.x) { tile_expert[i] = -1; tile_row[i] = 0; }
 }
 
-extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, int32_t* order, int32_t* offsets,
+extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, int tile_rows, int32_t* order, int32_t* offsets,
                            int32_t* tile_expert, int32_t* tile_row, hipStream_t stream) {
   if (P == 0) return 0;
   ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && P < (1ll << 30), "moe_sort: %d experts, %lld pairs", E, (long long)P);
-  ME_CHECK(max_tiles >= P / MOE_TM + (P < E ? P : E), "moe_sort: %d tiles cannot hold every expert's last tile", max_tiles);
-  moe_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, (int)P, E, max_tiles, order, offsets, tile_expert, tile_row);
+  ME_CHECK(tile_rows == 16 || tile_rows == MOE_TM, "moe_sort: tiles of 16 or %d rows", MOE_TM);
+  ME_CHECK(max_tiles >= P / tile_rows + (P < E ? P : E), "moe_sort: %d tiles cannot hold every expert's last tile", max_tiles);
+  moe_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, (int)P, E, max_tiles, tile_rows, order, offsets, tile_expert, tile_row);
   ME_LAUNCH_CHECK();
   return 0;
 }
@@ -319,14 +343,93 @@ moe_tile_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
   }
 }
 
+// ------------------------------------------------------------------ few rows per expert
+// Tiles of up to 16 pair rows (a decode step: a handful of tokens per expert). What such a step costs is the stream of
+// the chosen experts' weights, so a workgroup takes 16 features only and cuts K over its 4 waves: a wave walks every
+// fourth step of 32, its lanes asking memory for their operand pieces directly (no LDS on the way in), four steps in
+// flight; the waves' sums meet in LDS.
+template <bool ACT>
+__global__ void __launch_bounds__(256)
+moe_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
+                  const int32_t* __restrict__ offsets, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row,
+                  const float* __restrict__ pair_weight, void* __restrict__ out, int64_t T, int top, int N, int K) {
+  __shared__ float part[4][ACT ? 2 : 1][64][4];
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int row0 = tile_row[blockIdx.y];
+  const int rows = min(16, offsets[e + 1] - row0);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int p = row0 + min(n, rows - 1);
+  const bf16_t* xr = x + (ACT ? (int64_t)(order[p] / top) : (int64_t)p) * ldx + 8 * g;
+  const int f = min(n0 + n, N - 1);
+  const bf16_t* wr = w + ((int64_t)e * (ACT ? 2 : 1) * N + f) * K + 8 * g;
+  const bf16_t* ur = wr + (int64_t)N * K;            // ACT: the up row of the same feature
+  f32x4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = wave * 32; k0 < K; k0 += 4 * 128) {
+    bf16x8 a[4], u[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + i * 128;
+      const bool in = k + 8 * g < K;
+      a[i] = in ? *reinterpret_cast<const bf16x8*>(wr + k) : zero;
+      if (ACT) u[i] = in ? *reinterpret_cast<const bf16x8*>(ur + k) : zero;
+      b[i] = in ? *reinterpret_cast<const bf16x8*>(xr + k) : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[i], acc_g, 0, 0, 0);
+      if (ACT) acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[i], b[i], acc_u, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    part[wave][0][lane][q] = acc_g[q];
+    if (ACT) part[wave][1][lane][q] = acc_u[q];
+  }
+  __syncthreads();
+  if (wave != 0 || n >= rows) return;
+  // lane (n, g): features n0 + 4 g .. + 3 of pair row n
+  const int pr = row0 + n;
+  float sg[4], su[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    sg[q] = part[0][0][lane][q] + part[1][0][lane][q] + part[2][0][lane][q] + part[3][0][lane][q];
+    if (ACT) su[q] = part[0][1][lane][q] + part[1][1][lane][q] + part[2][1][lane][q] + part[3][1][lane][q];
+  }
+  if constexpr (ACT) {
+    bf16_t* o = (bf16_t*)out + (int64_t)pr * N;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (n0 + 4 * g + q < N) o[n0 + 4 * g + q] = from_f32<bf16_t>(sg[q] / (1.f + __expf(-sg[q])) * su[q]);
+  } else {
+    const int pair = order[pr];
+    const int64_t tok = pair / top, choice = pair - tok * top;
+    const float pw = pair_weight[pair];
+    float* o = (float*)out + (choice * T + tok) * N;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (n0 + 4 * g + q < N) o[n0 + 4 * g + q] = sg[q] * pw;
+  }
+}
+
 // act: bfloat16 [P, F] at sorted places; gate_up: [E * 2 F, K] (an expert's gate rows, then its up rows)
+// tile_rows: 16 (tiles of `moe_sort` with 16 rows: the skinny kernel) or 64
 extern "C" int me_moe_gate_up(const void* x, int64_t ldx, const void* gate_up, const int32_t* order, const int32_t* offsets,
                               const int32_t* tile_expert, const int32_t* tile_row, void* act, int64_t T, int top, int F, int K,
-                              int max_tiles, hipStream_t stream) {
+                              int max_tiles, int tile_rows, hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(K % 8 == 0 && ldx % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0,
            "moe_gate_up: rows must be whole 16-byte pieces (K = %d)", K);
   ME_CHECK(max_tiles >= 1 && max_tiles <= 65535 && F >= 1, "moe_gate_up: %d tiles", max_tiles);
+  if (tile_rows == 16) {
+    moe_skinny_kernel<true><<<dim3((unsigned)((F + 15) / 16), (unsigned)max_tiles), dim3(256), 0, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)gate_up, order, offsets, tile_expert, tile_row, nullptr, act, T, top, F, K);
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   moe_tile_kernel<true><<<dim3((unsigned)((F + 31) / 32), (unsigned)max_tiles), dim3(256), 0, stream>>>(
       (const bf16_t*)x, ldx, (const bf16_t*)gate_up, (int64_t)K, order, offsets, tile_expert, tile_row, nullptr, act, T, top, F, K);
   ME_LAUNCH_CHECK();
@@ -336,11 +439,17 @@ extern "C" int me_moe_gate_up(const void* x, int64_t ldx, const void* gate_up, c
 // out: float32 [top, T, N]; down: [E * N, F]
 extern "C" int me_moe_down(const void* act, const void* down, const int32_t* order, const int32_t* offsets,
                            const int32_t* tile_expert, const int32_t* tile_row, const float* pair_weight, float* out, int64_t T,
-                           int top, int N, int F, int max_tiles, hipStream_t stream) {
+                           int top, int N, int F, int max_tiles, int tile_rows, hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(F % 8 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0 && reinterpret_cast<uintptr_t>(down) % 16 == 0,
            "moe_down: rows must be whole 16-byte pieces (F = %d)", F);
   ME_CHECK(max_tiles >= 1 && max_tiles <= 65535 && N >= 1, "moe_down: %d tiles", max_tiles);
+  if (tile_rows == 16) {
+    moe_skinny_kernel<false><<<dim3((unsigned)((N + 15) / 16), (unsigned)max_tiles), dim3(256), 0, stream>>>(
+        (const bf16_t*)act, (int64_t)F, (const bf16_t*)down, order, offsets, tile_expert, tile_row, pair_weight, out, T, top, N, F);
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   moe_tile_kernel<false><<<dim3((unsigned)((N + 63) / 64), (unsigned)max_tiles), dim3(256), 0, stream>>>(
       (const bf16_t*)act, (int64_t)F, (const bf16_t*)down, (int64_t)F, order, offsets, tile_expert, tile_row, pair_weight, out, T, top, N, F);
   ME_LAUNCH_CHECK();

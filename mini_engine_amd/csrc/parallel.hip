@@ -23,34 +23,94 @@ struct SumTerms {
   int count;
 };
 
-// One workgroup per row; the row stays in LDS between the sum and the norms.
-template <typename TY>
-__global__ void scaled_sum_norm_kernel(const void* __restrict__ stream_in, int stream_dtype, SumTerms terms, float mult,
-                                       float* __restrict__ stream_out, const float* __restrict__ w1,
-                                       const float* __restrict__ w2, TY* __restrict__ y1, TY* __restrict__ y2, int n, float eps) {
+// One element of a term: its partial sums added in order, times the term's scale.
+__device__ __forceinline__ float term_value(const void* ptr, int dtype, int parts, int64_t stride, const float* scale,
+                                            int64_t at, int i) {
+  float v = 0.f;
+  if (dtype == ME_F32) {
+    const float* p = (const float*)ptr + at;
+    for (int q = 0; q < parts; ++q) v += p[q * stride];
+  } else {
+    const bf16_t* p = (const bf16_t*)ptr + at;
+    for (int q = 0; q < parts; ++q) v += static_cast<float>(p[q * stride]);
+  }
+  return scale ? scale[i] * v : v;
+}
+
+// The same for 4 neighbours (16-byte loads where the term is float32).
+__device__ __forceinline__ void term_value4(const void* ptr, int dtype, int parts, int64_t stride, const float* scale,
+                                            int64_t at, int i, float (&out)[4]) {
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (dtype == ME_F32) {
+    const float* p = (const float*)ptr + at;
+    for (int q = 0; q < parts; ++q) {
+      const float4 t = *reinterpret_cast<const float4*>(p + q * stride);
+      v[0] += t.x; v[1] += t.y; v[2] += t.z; v[3] += t.w;
+    }
+  } else {
+    const bf16_t* p = (const bf16_t*)ptr + at;
+    for (int q = 0; q < parts; ++q) {
+      const bf16x4 t = *reinterpret_cast<const bf16x4*>(p + q * stride);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] += static_cast<float>(t[j]);
+    }
+  }
+  float4 sc = make_float4(1.f, 1.f, 1.f, 1.f);
+  if (scale) sc = *reinterpret_cast<const float4*>(scale + i);
+  out[0] += sc.x * v[0]; out[1] += sc.y * v[1]; out[2] += sc.z * v[2]; out[3] += sc.w * v[3];
+}
+
+// One workgroup per row; the row stays in LDS between the sum and the norms. The terms are walked by a loop that the
+// compiler unrolls, so that their pointers stay in scalar registers. VEC: rows in whole groups of 4 with every operand
+// 16-byte aligned: a thread takes 4 neighbours at a time.
+template <typename TY, bool VEC>
+__global__ void __launch_bounds__(1024)
+scaled_sum_norm_kernel(const void* __restrict__ stream_in, int stream_dtype, SumTerms terms, float mult,
+                       float* __restrict__ stream_out, const float* __restrict__ w1, const float* __restrict__ w2,
+                       TY* __restrict__ y1, TY* __restrict__ y2, int n, float eps) {
   __shared__ float scratch[16];
-  extern __shared__ float row[];
+  extern __shared__ __align__(16) float row[];
   const int64_t t = blockIdx.x;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int64_t at = t * n + i;
-    float add = 0.f;
-    for (int k = 0; k < terms.count; ++k) {
-      float v = 0.f;
-      if (terms.dtype[k] == ME_F32) {
-        const float* p = (const float*)terms.ptr[k] + at;
-        for (int q = 0; q < terms.parts[k]; ++q) v += p[q * terms.part_stride[k]];
+  if constexpr (VEC) {
+    for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+      const int64_t at = t * n + i;
+      float add[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < PS_MAX_TERMS; ++k)
+        if (k < terms.count) term_value4(terms.ptr[k], terms.dtype[k], terms.parts[k], terms.part_stride[k], terms.scale[k], at, i, add);
+      float base[4];
+      if (stream_dtype == ME_F32) {
+        const float4 b = *reinterpret_cast<const float4*>((const float*)stream_in + at);
+        base[0] = b.x; base[1] = b.y; base[2] = b.z; base[3] = b.w;
       } else {
-        const bf16_t* p = (const bf16_t*)terms.ptr[k] + at;
-        for (int q = 0; q < terms.parts[k]; ++q) v += static_cast<float>(p[q * terms.part_stride[k]]);
+        const bf16x4 b = *reinterpret_cast<const bf16x4*>((const bf16_t*)stream_in + at);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) base[j] = static_cast<float>(b[j]);
       }
-      add += terms.scale[k] ? terms.scale[k][i] * v : v;
+      float s[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s[j] = terms.count ? base[j] + mult * add[j] : base[j];
+        ss += s[j] * s[j];
+      }
+      const float4 out = make_float4(s[0], s[1], s[2], s[3]);
+      if (stream_out) *reinterpret_cast<float4*>(stream_out + at) = out;
+      *reinterpret_cast<float4*>(row + i) = out;
     }
-    const float base = stream_dtype == ME_F32 ? ((const float*)stream_in)[at] : static_cast<float>(((const bf16_t*)stream_in)[at]);
-    const float s = terms.count ? base + mult * add : base;
-    if (stream_out) stream_out[at] = s;
-    row[i] = s;
-    ss += s * s;
+  } else {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int64_t at = t * n + i;
+      float add = 0.f;
+#pragma unroll
+      for (int k = 0; k < PS_MAX_TERMS; ++k)
+        if (k < terms.count) add += term_value(terms.ptr[k], terms.dtype[k], terms.parts[k], terms.part_stride[k], terms.scale[k], at, i);
+      const float base = stream_dtype == ME_F32 ? ((const float*)stream_in)[at] : static_cast<float>(((const bf16_t*)stream_in)[at]);
+      const float s = terms.count ? base + mult * add : base;
+      if (stream_out) stream_out[at] = s;
+      row[i] = s;
+      ss += s * s;
+    }
   }
   if (!w1) return;
   ss = block_sum(ss, scratch);
@@ -85,14 +145,25 @@ extern "C" int me_scaled_sum_norm(const void* stream_in, int stream_dtype, int c
     ME_CHECK(!on || (terms.parts[k] >= 1 && terms.parts[k] <= 64), "scaled_sum_norm: 1 to 64 partial sums per term");
     ME_CHECK(!on || terms.parts[k] == 1 || terms.dtype[k] == ME_F32, "scaled_sum_norm: partial sums are float32");
   }
-  const int threads = n >= 1024 ? 256 : (n > 256 ? 128 : 64);
+  // whole groups of 4 and every operand 16-byte aligned (a bfloat16 group is 8 bytes): the vector form
+  uintptr_t bits = reinterpret_cast<uintptr_t>(stream_in) | reinterpret_cast<uintptr_t>(stream_out);
+  bool vec = n % 4 == 0;
+  for (int k = 0; k < count; ++k) {
+    bits |= reinterpret_cast<uintptr_t>(terms.ptr[k]) | reinterpret_cast<uintptr_t>(terms.scale[k]);
+    vec = vec && terms.part_stride[k] % 4 == 0;
+  }
+  vec = vec && bits % 16 == 0;
+  // few rows: a row's threads are all the launch has, so as many as its groups fill; many rows: 256
+  const int per = vec ? 4 : 1;
+  int threads = T >= 512 ? 256 : 1024;
+  while (threads > 64 && threads * per / 2 >= n) threads >>= 1;
   const size_t lds = (size_t)n * sizeof(float);
-  if (out_dtype == ME_F32)
-    scaled_sum_norm_kernel<float><<<dim3((unsigned)T), dim3(threads), lds, stream>>>(stream_in, stream_dtype, terms, mult, stream_out,
-                                                                                  w1, w2, (float*)y1, (float*)y2, n, eps);
-  else
-    scaled_sum_norm_kernel<bf16_t><<<dim3((unsigned)T), dim3(threads), lds, stream>>>(stream_in, stream_dtype, terms, mult, stream_out,
-                                                                                   w1, w2, (bf16_t*)y1, (bf16_t*)y2, n, eps);
+#define PS_LAUNCH(TY, V)                                                                                                   \
+  scaled_sum_norm_kernel<TY, V><<<dim3((unsigned)T), dim3(threads), lds, stream>>>(stream_in, stream_dtype, terms, mult, stream_out, \
+                                                                                w1, w2, (TY*)y1, (TY*)y2, n, eps)
+  if (out_dtype == ME_F32) { if (vec) PS_LAUNCH(float, true); else PS_LAUNCH(float, false); }
+  else { if (vec) PS_LAUNCH(bf16_t, true); else PS_LAUNCH(bf16_t, false); }
+#undef PS_LAUNCH
   ME_LAUNCH_CHECK();
   return 0;
 }
@@ -124,7 +195,7 @@ extern "C" int me_softcap(float* z, int64_t ld, int64_t rows, int n, float cap, 
 //      mix 2: v <- (1 - lambda) v + lambda v_first; into the (transposed) page
 // K [pages, Hkv, page, D], V [pages, Hkv, D, page]; slots < 0 are skipped.
 template <typename TY>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 qkv_prepare_kernel(const float* __restrict__ rows, int64_t row_stride, const float* __restrict__ bias,
                    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, int nq, int nk,
                    float temp_coef, int temp_every, const int32_t* __restrict__ positions,
@@ -187,12 +258,15 @@ extern "C" int me_qkv_prepare(const float* rows, int64_t row_stride, const float
   ME_CHECK(mix >= 0 && mix <= 2 && (!mix || (v_first && vdim >= 1 && vdim <= D)) && (mix != 2 || lambda), "qkv_prepare: bad value mixing");
   ME_CHECK(temp_every >= 0, "qkv_prepare: bad temperature period");
   const size_t lds = (size_t)(Hq + Hkv) * D * sizeof(float);
+  // few tokens: a token's threads are all the launch has
+  int threads = T >= 512 ? 256 : 1024;
+  while (threads > 64 && threads / 2 >= (Hq + Hkv) * D) threads >>= 1;
   if (dtype == ME_F32)
-    qkv_prepare_kernel<float><<<dim3((unsigned)T), dim3(256), lds, stream>>>(
+    qkv_prepare_kernel<float><<<dim3((unsigned)T), dim3(threads), lds, stream>>>(
         rows, row_stride, bias, q_w, k_w, eps, nq, nk, temp_coef, temp_every, positions, slots, (float*)k_cache, (float*)v_cache,
         (float*)q_out, q_stride, Hq, Hkv, D, page, vdim, mix, lambda, v_first, vf_stride);
   else
-    qkv_prepare_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), lds, stream>>>(
+    qkv_prepare_kernel<bf16_t><<<dim3((unsigned)T), dim3(threads), lds, stream>>>(
         rows, row_stride, bias, q_w, k_w, eps, nq, nk, temp_coef, temp_every, positions, slots, (bf16_t*)k_cache, (bf16_t*)v_cache,
         (bf16_t*)q_out, q_stride, Hq, Hkv, D, page, vdim, mix, lambda, v_first, vf_stride);
   ME_LAUNCH_CHECK();

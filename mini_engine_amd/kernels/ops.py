@@ -80,10 +80,10 @@ _CORE_PROTOS = {
     "me_scaled_sum_norm": [P, I, I, P, P, P, P, P, F, P, P, P, P, P, I, L, I, F, P],
     "me_softcap": [P, L, L, I, F, P],
     "me_qkv_prepare": [P, L, P, P, P, F, I, I, F, I, P, P, P, P, P, L, I, L, I, I, I, I, I, I, P, P, L, P],
-    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P],
-    "me_moe_sort": [P, L, I, I, P, P, P, P, P],
-    "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, P],
-    "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, P],
+    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P, P],
+    "me_moe_sort": [P, L, I, I, I, P, P, P, P, P],
+    "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, P],
+    "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
@@ -790,16 +790,19 @@ class HipBackend:
                "moe_route: rows [T, n], router float32 [E, n]")
         ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
         weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+        logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
-                    int(group_keep), ids.data_ptr(), weights.data_ptr(), _stream())
+                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), _stream())
         return ids, weights
 
-    def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False) -> torch.Tensor:
+    def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False, tile_rows: int | None = None) -> torch.Tensor:
         """Every token through its chosen gated experts: out[j, t] = weights[t, j] * W_down[e] (silu(W_gate[e] x_t) * (W_up[e] x_t)),
         e = ids[t, j]: float32 [top, T, hidden], one partial sum per choice for a consumer that adds them. x: [T, K];
         gate_up: [E, 2 F, K] (an expert's gate rows, then its up rows); down: [E, hidden, F]. bfloat16 with K and F in
-        whole steps of 8: the (token, choice) pairs are ordered by expert and cut into tiles of 64 rows, each tile one
-        workgroup of the matrix-core kernels; otherwise (float32, other sizes) one wave per output element."""
+        whole steps of 8: the (token, choice) pairs are ordered by expert and cut into tiles that never span two experts, of
+        64 rows (a workgroup's 64 x 64 tile of the matrix-core kernel) or, while an expert gets few rows (`expert_tile_rows`;
+        `tile_rows` forces it), of 16 rows for the kernel that streams the chosen experts' weights with K cut over a
+        workgroup's waves; otherwise (float32, other sizes) one wave per output element."""
         T, K = x.shape
         top = ids.shape[1]
         E, F2, _ = gate_up.shape
@@ -811,22 +814,23 @@ class HipBackend:
         out = torch.empty((top, T, N), dtype=torch.float32, device=x.device)
         Pn = T * top
         act = torch.empty((Pn, F), dtype=x.dtype, device=x.device)
+        rows = tile_rows or expert_tile_rows(T, top, E)
         tiled = (x.dtype == torch.bfloat16 and K % 8 == 0 and F % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-                 and not force_simple and Pn // 64 + min(E, Pn) <= 65535)
+                 and not force_simple and Pn // rows + min(E, Pn) <= 65535)
         if not tiled:
             core().call("me_moe_experts_simple", x.data_ptr(), x.stride(0), _code(x.dtype), gate_up.data_ptr(), down.data_ptr(),
                         ids.data_ptr(), weights.data_ptr(), act.data_ptr(), out.data_ptr(), T, top, N, F, K, _stream())
             return out
-        max_tiles = Pn // 64 + min(E, Pn)
+        max_tiles = Pn // rows + min(E, Pn)
         meta = torch.empty((Pn + E + 1 + 2 * max_tiles,), dtype=torch.int32, device=x.device)
         order, offsets = meta[:Pn], meta[Pn:Pn + E + 1]
         tile_expert, tile_row = meta[Pn + E + 1:Pn + E + 1 + max_tiles], meta[Pn + E + 1 + max_tiles:]
-        core().call("me_moe_sort", ids.data_ptr(), Pn, E, max_tiles, order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
+        core().call("me_moe_sort", ids.data_ptr(), Pn, E, max_tiles, rows, order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
                     tile_row.data_ptr(), _stream())
         core().call("me_moe_gate_up", x.data_ptr(), x.stride(0), gate_up.data_ptr(), order.data_ptr(), offsets.data_ptr(),
-                    tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, _stream())
+                    tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, rows, _stream())
         core().call("me_moe_down", act.data_ptr(), down.data_ptr(), order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
-                    tile_row.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, N, F, max_tiles, _stream())
+                    tile_row.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, N, F, max_tiles, rows, _stream())
         return out
 
     # -- sampling ------------------------------------------------------------------------
@@ -1287,6 +1291,17 @@ def recurrence_spans(q_lens: list, waves_per_request: int, most_spans: int = 819
     span = -(-span // 16) * 16
     spans = -(-longest // span)
     return (span, spans) if spans >= 2 else (0, 1)
+
+
+EXPERT_SKINNY_MAX_ROWS = 24       # mean rows per expert up to which the 16-row tiles of the streaming kernel are taken
+
+
+def expert_tile_rows(T: int, top: int, E: int) -> int:
+    """Rows per tile of the routed experts' kernels: 16 while an expert gets EXPERT_SKINNY_MAX_ROWS rows or fewer on
+    average (decode steps and short portions: the step is the stream of the chosen experts' weights, and a tile of 16
+    rows reads an expert's weights once per 16 rows with K cut over a workgroup's waves), else 64 (the tiles of the
+    matrix-core kernel that stages its operands in LDS)."""
+    return 16 if T * top <= EXPERT_SKINNY_MAX_ROWS * E else 64
 
 
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:

@@ -321,7 +321,7 @@ def moe_route(x, router, top, group_count=1, group_keep=1):
     return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20)).float()
 
 
-def routed_experts(x, ids, weights, gate_up, down, force_simple=False):
+def routed_experts(x, ids, weights, gate_up, down, force_simple=False, tile_rows=None):
     T, K = x.shape
     top = ids.shape[1]
     F = gate_up.shape[1] // 2
