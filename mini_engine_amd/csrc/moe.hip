@@ -3,7 +3,7 @@
 //   moe_route      float32 router: logits = W x, softmax over all experts, optionally only the experts of the best
 //                  groups of neighbours stay eligible (a group scores as its best expert), the `top` largest scores
 //                  are chosen and divided by their sum
-//   moe_sort       (token, choice) pairs ordered by expert, cut into tiles of 64 rows that never span two experts
+//   moe_sort       (token, choice) pairs ordered by expert, cut into tiles of 16, 64 or 128 rows that never span two experts
 //   moe_gate_up    per tile: silu(x W_gate^T) * (x W_up^T) of the tile's expert, token rows gathered through the order
 //   moe_down       per tile: the expert's down product, times the pair's weight, into float32 [top, T, hidden]: one
 //                  partial sum per choice, for a consumer that adds them (no atomics: the result does not depend on
@@ -11,7 +11,7 @@
 //   moe_*_simple   the same two products with one wave per output element: the float32 path, and sizes whose rows
 //                  are not whole 16-byte pieces
 //
-// The tiled kernels: a workgroup owns 64 pair rows x 64 weight rows, its 4 waves 2 x 2 sub-tiles of 32 x 32
+// The tiled kernels: a workgroup owns 64 pair rows x 64 weight rows (or 128 x 128), its 4 waves 2 x 2 sub-tiles
 // (v_mfma_f32_16x16x32_bf16, weight rows as the A operand, so that a lane holds 4 consecutive features of one
 // row); K is walked 64 at a time through two LDS buffers, the next step's 16-byte pieces on their way in registers
 // while the current one is multiplied; piece c of row R lies at c ^ (R >> 1 & 7), so that the 16 lanes of an operand
@@ -35,6 +35,17 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
     const int oi = __shfl_xor(i, off, ME_WAVE);
     if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
   }
+}
+
+// Four neighbours of a row as float32 (one 8- or 16-byte read).
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&v)[4]) {
+  const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = static_cast<float>(t[j]);
 }
 
 // Router logits: a workgroup of 4 waves takes `tokens_per_group` tokens (their rows wait in LDS) and `experts_per_group`
@@ -68,8 +79,9 @@ moe_logits_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict
 #pragma unroll
         for (int tt = 0; tt < 8; ++tt)
           if (tt < TT) {
-            const TX* xr = xs + tt * n + k;
-            acc[tt] += wv.x * to_f32<TX>(xr[0]) + wv.y * to_f32<TX>(xr[1]) + wv.z * to_f32<TX>(xr[2]) + wv.w * to_f32<TX>(xr[3]);
+            float xv[4];
+            load4(xs + tt * n + k, xv);
+            acc[tt] += wv.x * xv[0] + wv.y * xv[1] + wv.z * xv[2] + wv.w * xv[3];
           }
       }
     } else {
@@ -216,7 +228,7 @@ extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, 
                            int32_t* tile_expert, int32_t* tile_row, hipStream_t stream) {
   if (P == 0) return 0;
   ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && P < (1ll << 30), "moe_sort: %d experts, %lld pairs", E, (long long)P);
-  ME_CHECK(tile_rows == 16 || tile_rows == MOE_TM, "moe_sort: tiles of 16 or %d rows", MOE_TM);
+  ME_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_sort: tiles of 16, 64 or 128 rows");
   ME_CHECK(max_tiles >= P / tile_rows + (P < E ? P : E), "moe_sort: %d tiles cannot hold every expert's last tile", max_tiles);
   moe_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, (int)P, E, max_tiles, tile_rows, order, offsets, tile_expert, tile_row);
   ME_LAUNCH_CHECK();
@@ -224,123 +236,142 @@ extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, 
 }
 
 // ------------------------------------------------------------------ tiled products
-// A stage in LDS: 64 B rows (pairs) then 64 A rows (weights), 128 bytes each.
-struct MoeStage {
-  uint4 piece[4];
-};
-
-// ACT: the tile's weight rows are 32 gate rows and the 32 up rows that go with them; the result is silu(gate) * up.
+// A stage in LDS: TM B rows (pairs) then TN A rows (weights), 128 bytes each. A workgroup's 4 waves are 2 x 2
+// sub-tiles of TM/2 x TN/2, each MJ x MI matrix-instruction tiles of 16 x 16: 64 x 64 (2 x 2 per wave) for a few
+// hundred rows per expert, 128 x 128 (4 x 4 per wave: twice the products per operand read from LDS) beyond.
+// ACT: the tile's weight rows are TN/2 gate rows and the TN/2 up rows that go with them; the result is silu(gate) * up.
 //   x: [T, K] token rows (ACT) or [P, K] rows at sorted places; w: [E * rows_per_expert, K]
-template <bool ACT>
+template <bool ACT, int TM, int TN>
 __global__ void __launch_bounds__(256)
 moe_tile_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                 const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const int32_t* __restrict__ tile_expert,
                 const int32_t* __restrict__ tile_row, const float* __restrict__ pair_weight, void* __restrict__ out,
                 int64_t T, int top, int N, int K) {
-  __shared__ __align__(16) unsigned char lds[2][128 * 128];
+  constexpr int ROWS = TM + TN, NQ = ROWS / 32, MI = TN / 32, MJ = TM / 32, STAGE = ROWS * 128;
+  extern __shared__ __align__(16) unsigned char lds[];        // [2][STAGE]
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   const int row0 = tile_row[blockIdx.y];
-  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  const int rows = min(TM, offsets[e + 1] - row0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (ACT ? 32 : 64);           // first feature of the tile
-  // the 4 pieces this thread brings per stage: rows tid / 8 + 32 q, piece tid % 8
-  const bf16_t* src[4];
-  uint32_t dst[4];
+  const int n0 = blockIdx.x * (ACT ? TN / 2 : TN);           // first feature of the tile
+  // the pieces this thread brings per stage: rows tid / 8 + 32 q, piece tid % 8
+  const bf16_t* src[NQ];
+  uint32_t dst[NQ];
   const int c = tid & 7;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int R = (tid >> 3) + 32 * q;
-    if (R < MOE_TM) {
+    if (R < TM) {
       const int p = row0 + min(R, rows - 1);
       const int64_t from = ACT ? (int64_t)(order[p] / top) : (int64_t)p;
       src[q] = x + from * ldx;
     } else {
-      const int wr = R - MOE_TM;
+      const int wr = R - TM;
       int64_t row;
-      if (ACT) row = (int64_t)e * 2 * N + (wr < 32 ? min(n0 + wr, N - 1) : N + min(n0 + wr - 32, N - 1));
+      if (ACT) row = (int64_t)e * 2 * N + (wr < TN / 2 ? min(n0 + wr, N - 1) : N + min(n0 + wr - TN / 2, N - 1));
       else row = (int64_t)e * N + min(n0 + wr, N - 1);
       src[q] = w + row * ldw;
     }
     dst[q] = R * 128 + ((c ^ ((R >> 1) & 7)) * 16);
   }
-  auto fetch = [&](int k0, MoeStage& st) {
+  uint4 piece[NQ];
+  auto fetch = [&](int k0) {
+    const int k = k0 + 8 * c;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int k = k0 + 8 * c;
-      st.piece[q] = k < K ? *reinterpret_cast<const uint4*>(src[q] + k) : make_uint4(0u, 0u, 0u, 0u);
-    }
+    for (int q = 0; q < NQ; ++q) piece[q] = k < K ? *reinterpret_cast<const uint4*>(src[q] + k) : make_uint4(0u, 0u, 0u, 0u);
   };
-  auto put = [&](int b, const MoeStage& st) {
+  auto put = [&](int b) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4*>(&lds[b][dst[q]]) = st.piece[q];
+    for (int q = 0; q < NQ; ++q) *reinterpret_cast<uint4*>(lds + b * STAGE + dst[q]) = piece[q];
   };
   const int wm = wave >> 1, wn = wave & 1;
   const int swz = (n >> 1) & 7;
-  uint32_t rd_b[2], rd_a[2];
+  // rows of the wave's operand tiles: pairs wm * TM/2 + 16 j + n; weights (ACT: half of them gates, half their ups)
+  int a_row[MI];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    rd_b[s] = (wm * 32 + n) * 128 + (((4 * s + g) ^ swz) * 16);
-    rd_a[s] = (MOE_TM + wn * (ACT ? 16 : 32) + n) * 128 + (((4 * s + g) ^ swz) * 16);
-  }
-  f32x4 acc[2][2];
+  for (int i = 0; i < MI; ++i)
+    a_row[i] = TM + (ACT ? (i < MI / 2 ? wn * (TN / 4) + 16 * i : TN / 2 + wn * (TN / 4) + 16 * (i - MI / 2)) : wn * (TN / 2) + 16 * i) + n;
+  f32x4 acc[MI][MJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < MJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int steps = (K + 63) / 64;
-  MoeStage st;
-  fetch(0, st);
-  put(0, st);
+  fetch(0);
+  put(0);
   __syncthreads();
   for (int k = 0; k < steps; ++k) {
-    if (k + 1 < steps) fetch((k + 1) * 64, st);
-    const unsigned char* buf = lds[k & 1];
+    if (k + 1 < steps) fetch((k + 1) * 64);
+    const unsigned char* buf = lds + (k & 1) * STAGE;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      bf16x8 a[2], b[2];
+      const int col = ((4 * s + g) ^ swz) * 16;
+      bf16x8 a[MI], b[MJ];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + (ACT ? 32 : 16) * 128 * i);
+      for (int i = 0; i < MI; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + a_row[i] * 128 + col);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + rd_b[s] + 16 * 128 * j);
+      for (int j = 0; j < MJ; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + (wm * (TM / 2) + 16 * j + n) * 128 + col);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < MJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    if (k + 1 < steps) put((k + 1) & 1, st);
+    if (k + 1 < steps) put((k + 1) & 1);
     __syncthreads();
   }
-  // lane (n, g) of tile (i, j): features ... + 4 g .. + 3 of pair row 32 wm + 16 j + n
+  // lane (n, g) of tile (i, j): 4 consecutive features from 4 g of pair row wm * TM/2 + 16 j + n
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int r = wm * 32 + 16 * j + n;
+  for (int j = 0; j < MJ; ++j) {
+    const int r = wm * (TM / 2) + 16 * j + n;
     if (r >= rows) continue;
     const int p = row0 + r;
     if constexpr (ACT) {
       bf16_t* o = (bf16_t*)out + (int64_t)p * N;
-      const int f = n0 + wn * 16 + 4 * g;
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (f + q < N) {
-          const float gate = acc[0][j][q];
-          o[f + q] = from_f32<bf16_t>(gate / (1.f + __expf(-gate)) * acc[1][j][q]);
-        }
+      for (int i = 0; i < MI / 2; ++i) {
+        const int f = n0 + wn * (TN / 4) + 16 * i + 4 * g;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (f + q < N) {
+            const float gate = acc[i][j][q];
+            o[f + q] = from_f32<bf16_t>(gate / (1.f + __expf(-gate)) * acc[i + MI / 2][j][q]);
+          }
+      }
     } else {
       const int pair = order[p];
       const int64_t tok = pair / top, choice = pair - tok * top;
       const float pw = pair_weight[pair];
       float* o = (float*)out + (choice * T + tok) * N;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int f = n0 + wn * 32 + 16 * i + 4 * g;
+      for (int i = 0; i < MI; ++i) {
+        const int f = n0 + wn * (TN / 2) + 16 * i + 4 * g;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           if (f + q < N) o[f + q] = acc[i][j][q] * pw;
       }
     }
   }
+}
+
+template <bool ACT, int TM>
+static int launch_moe_tile(const bf16_t* x, int64_t ldx, const bf16_t* w, int64_t ldw, const int32_t* order, const int32_t* offsets,
+                           const int32_t* tile_expert, const int32_t* tile_row, const float* pair_weight, void* out, int64_t T,
+                           int top, int N, int K, int max_tiles, hipStream_t stream) {
+  constexpr int TN = TM;
+  const size_t lds = 2 * (size_t)(TM + TN) * 128;
+  static bool allowed = false;                     // 64 KB of LDS for the large tiles: more than a kernel may have unasked
+  if (!allowed && lds > 48 * 1024) {
+    hipError_t err = hipFuncSetAttribute((const void*)moe_tile_kernel<ACT, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ME_CHECK(err == hipSuccess, "routed experts: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+    allowed = true;
+  }
+  const int per = ACT ? TN / 2 : TN;
+  moe_tile_kernel<ACT, TM, TN><<<dim3((unsigned)((N + per - 1) / per), (unsigned)max_tiles), dim3(256), lds, stream>>>(
+      x, ldx, w, ldw, order, offsets, tile_expert, tile_row, pair_weight, out, T, top, N, K);
+  ME_LAUNCH_CHECK();
+  return 0;
 }
 
 // ------------------------------------------------------------------ few rows per expert
@@ -430,10 +461,12 @@ extern "C" int me_moe_gate_up(const void* x, int64_t ldx, const void* gate_up, c
     ME_LAUNCH_CHECK();
     return 0;
   }
-  moe_tile_kernel<true><<<dim3((unsigned)((F + 31) / 32), (unsigned)max_tiles), dim3(256), 0, stream>>>(
-      (const bf16_t*)x, ldx, (const bf16_t*)gate_up, (int64_t)K, order, offsets, tile_expert, tile_row, nullptr, act, T, top, F, K);
-  ME_LAUNCH_CHECK();
-  return 0;
+  if (tile_rows == 128)
+    return launch_moe_tile<true, 128>((const bf16_t*)x, ldx, (const bf16_t*)gate_up, (int64_t)K, order, offsets, tile_expert, tile_row,
+                                      nullptr, act, T, top, F, K, max_tiles, stream);
+  ME_CHECK(tile_rows == 64, "moe_gate_up: tiles of 16, 64 or 128 rows");
+  return launch_moe_tile<true, 64>((const bf16_t*)x, ldx, (const bf16_t*)gate_up, (int64_t)K, order, offsets, tile_expert, tile_row,
+                                   nullptr, act, T, top, F, K, max_tiles, stream);
 }
 
 // out: float32 [top, T, N]; down: [E * N, F]
@@ -450,10 +483,12 @@ extern "C" int me_moe_down(const void* act, const void* down, const int32_t* ord
     ME_LAUNCH_CHECK();
     return 0;
   }
-  moe_tile_kernel<false><<<dim3((unsigned)((N + 63) / 64), (unsigned)max_tiles), dim3(256), 0, stream>>>(
-      (const bf16_t*)act, (int64_t)F, (const bf16_t*)down, (int64_t)F, order, offsets, tile_expert, tile_row, pair_weight, out, T, top, N, F);
-  ME_LAUNCH_CHECK();
-  return 0;
+  if (tile_rows == 128)
+    return launch_moe_tile<false, 128>((const bf16_t*)act, (int64_t)F, (const bf16_t*)down, (int64_t)F, order, offsets, tile_expert,
+                                       tile_row, pair_weight, out, T, top, N, F, max_tiles, stream);
+  ME_CHECK(tile_rows == 64, "moe_down: tiles of 16, 64 or 128 rows");
+  return launch_moe_tile<false, 64>((const bf16_t*)act, (int64_t)F, (const bf16_t*)down, (int64_t)F, order, offsets, tile_expert,
+                                    tile_row, pair_weight, out, T, top, N, F, max_tiles, stream);
 }
 
 // ------------------------------------------------------------------ one wave per output element

@@ -1294,14 +1294,18 @@ def recurrence_spans(q_lens: list, waves_per_request: int, most_spans: int = 819
 
 
 EXPERT_SKINNY_MAX_ROWS = 24       # mean rows per expert up to which the 16-row tiles of the streaming kernel are taken
+EXPERT_LARGE_TILE_ROWS = 160      # ... from which tiles of 128 x 128 are taken
 
 
 def expert_tile_rows(T: int, top: int, E: int) -> int:
     """Rows per tile of the routed experts' kernels: 16 while an expert gets EXPERT_SKINNY_MAX_ROWS rows or fewer on
     average (decode steps and short portions: the step is the stream of the chosen experts' weights, and a tile of 16
     rows reads an expert's weights once per 16 rows with K cut over a workgroup's waves), else 64 (the tiles of the
-    matrix-core kernel that stages its operands in LDS)."""
-    return 16 if T * top <= EXPERT_SKINNY_MAX_ROWS * E else 64
+    matrix-core kernel that stages its operands in LDS), and 128 from EXPERT_LARGE_TILE_ROWS rows per expert on (tiles of
+    128 x 128: twice the products per operand read from LDS; below, too many of their rows would be empty)."""
+    if T * top <= EXPERT_SKINNY_MAX_ROWS * E:
+        return 16
+    return 128 if T * top >= EXPERT_LARGE_TILE_ROWS * E else 64
 
 
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:

@@ -112,11 +112,11 @@ def test_router(dtype, E, top, count, keep, n):
             assert all(len({e // per for e in row}) <= keep for row in ids.tolist())
 
 
-@pytest.mark.parametrize("dtype,simple", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, 16), (torch.bfloat16, 64)])
+@pytest.mark.parametrize("dtype,simple", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, 16), (torch.bfloat16, 64), (torch.bfloat16, 128)])
 @pytest.mark.parametrize("E,top,F,K,T", [(12, 2, 48, 160, 45), (4, 1, 40, 72, 300), (8, 3, 200, 136, 1), (32, 4, 256, 512, 700), (5, 5, 24, 64, 3),
                                           (64, 6, 1408, 2048, 130)])
 def test_routed_experts(dtype, simple, E, top, F, K, T):
-    """The kernels on tiles of 64 rows, on tiles of 16 rows, and the one-wave-per-element kernels against the plain loop: experts without tokens, experts with
+    """The kernels on tiles of 128, 64 and 16 rows, and the one-wave-per-element kernels against the plain loop: experts without tokens, experts with
     more than one tile, one token, sizes that are no multiples of the tiles."""
     torch.manual_seed(E * top + T)
     x = torch.randn(T, K, device=DEV).to(dtype)
