@@ -159,7 +159,21 @@ def _is_i32(t: torch.Tensor, n: int | None = None) -> bool:
 # --------------------------------------------------------------------------- the HIP backend
 
 LIBRARY_WORKSPACE_BYTES = 64 << 20
-_library_workspace: torch.Tensor | None = None
+_library_workspaces: dict = {}            # slot -> workspace: products that run side by side on two streams must not share one
+_workspace_slot = 0
+
+
+class second_workspace:
+    """While this is entered, library products use a workspace of their own: for work launched on a second stream beside
+    the main one."""
+
+    def __enter__(self):
+        global _workspace_slot
+        self.before, _workspace_slot = _workspace_slot, 1
+
+    def __exit__(self, *exc):
+        global _workspace_slot
+        _workspace_slot = self.before
 _library_direct: bool | None = None      # None: not asked yet
 
 
@@ -191,16 +205,17 @@ def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, sp
     splits > 1: K is cut in that many equal slices, computed as one strided batch; the result is their
     float32 partial sums [splits, M, N] for a consumer that adds them, or None where only torch's
     route is open (the caller then takes its other path)."""
-    global _library_workspace
+    handle = _stream()
+    _library_workspace = _library_workspaces.get(_workspace_slot)
     if library_is_direct() and _library_workspace is None and not torch.cuda.is_current_stream_capturing():
-        _library_workspace = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+        _library_workspace = _library_workspaces[_workspace_slot] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
     if _library_direct and _library_workspace is not None:
         M, K = x.shape
         N = w.shape[0]
         y = out if out is not None else torch.empty((M, N) if splits == 1 else (splits, M, N), dtype=out_dtype, device=x.device)
         rc = core().fns["me_gemm_library_bf16"](x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                                                _code(out_dtype), _library_workspace.data_ptr(),
-                                               LIBRARY_WORKSPACE_BYTES, M, N, K, splits, _stream())
+                                               LIBRARY_WORKSPACE_BYTES, M, N, K, splits, handle)
         if rc == 0:
             return y
         if rc != -3:

@@ -766,7 +766,7 @@ def test_library_product_is_called_directly(M, N, K):
     w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
     ref = x.double() @ w.double().t()
     close(ops.library_product(x, w, torch.bfloat16), ref, 6e-3)
-    assert ops._library_direct is True and ops._library_workspace is not None
+    assert ops._library_direct is True and ops._library_workspaces.get(0) is not None
     close(ops.library_product(x, w, torch.float32), ref, 2e-5)
     xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]
     close(ops.library_product(xs, w, torch.bfloat16), xs.double() @ w.double().t(), 6e-3)
