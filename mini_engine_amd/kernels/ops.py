@@ -167,9 +167,12 @@ class second_workspace:
     """While this is entered, library products use a workspace of their own: for work launched on a second stream beside
     the main one."""
 
+    def __init__(self, slot: int = 1):
+        self.slot = slot
+
     def __enter__(self):
         global _workspace_slot
-        self.before, _workspace_slot = _workspace_slot, 1
+        self.before, _workspace_slot = _workspace_slot, self.slot
 
     def __exit__(self, *exc):
         global _workspace_slot

@@ -250,6 +250,46 @@ class ScaledSum:
         return ops.scaled_sum_norm(stream, self.terms, self.mult, None, None, 0.0, torch.float32)[0]
 
 
+# Steps of up to this many tokens are chains of short launches: parts that have independent work then put it on further
+# streams (0: never). The streams have the default priority; a captured step holds such work as branches of its graph.
+SIDE_BRANCH_MAX_TOKENS = 64
+_side_streams: dict = {}
+
+
+class side_branch:
+    """`with side_branch(device, slot):` what is launched inside runs on a further stream (one per device and slot) that
+    starts behind everything launched so far on the current stream; `join()` afterwards makes the current stream wait
+    for it. Library products inside use a workspace of their own. What the branch allocates may be read on the current
+    stream only behind `join()`; the caller sees to it that it is not written again before its reader has been
+    launched (a later branch of the same slot starts behind whatever was launched before it)."""
+
+    def __init__(self, device: torch.device, slot: int = 1):
+        from ..kernels import ops
+        key = (device.type, device.index, slot)
+        if key not in _side_streams:
+            _side_streams[key] = torch.cuda.Stream(device=device)
+        self.stream, self.main = _side_streams[key], torch.cuda.current_stream(device)
+        self._inner = (torch.cuda.stream(self.stream), ops.second_workspace(slot))
+
+    def __enter__(self):
+        self.stream.wait_stream(self.main)
+        for c in self._inner:
+            c.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        for c in reversed(self._inner):
+            c.__exit__(*exc)
+
+    def join(self) -> None:
+        self.main.wait_stream(self.stream)
+
+
+def few_tokens(x: torch.Tensor) -> bool:
+    """Whether a step with rows x is one whose independent work goes to side branches."""
+    return x.is_cuda and 0 < x.shape[0] <= SIDE_BRANCH_MAX_TOKENS
+
+
 class PositionEncoding(Part):
     """Something applied to queries and keys as a function of token positions."""
 

@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import FeedForward, Mixer, Norm, ParamSpec, Part, PendingNorm, ScaledSum, Settled, register_part
+from .base import FeedForward, Mixer, Norm, ParamSpec, Part, PendingNorm, ScaledSum, Settled, few_tokens, register_part, side_branch
 
 
 def one_tensor(x):
@@ -115,19 +115,6 @@ class OutputNormBlock(Part):
         return Settled(x), stream
 
 
-SIDE_BRANCH_MAX_TOKENS = 64      # steps of up to this many tokens run a parallel block's two sublayers on two streams (0: never)
-_side_streams: dict = {}
-
-
-def _side_stream(device):
-    """One further stream per device, of the default priority, for the second sublayer of parallel blocks."""
-    import torch
-    key = (device.type, device.index)
-    if key not in _side_streams:
-        _side_streams[key] = torch.cuda.Stream(device=device)
-    return _side_streams[key]
-
-
 def _ones(shape, generator, device):
     import torch
     return 1.0 + 0.2 * (torch.rand(shape, generator=generator, dtype=torch.float32, device=device) - 0.5)
@@ -142,10 +129,10 @@ class ParallelBlock(Part):
     layer before has left (`ScaledSum`), so a stack of such layers costs one pass over the stream per layer. The
     stream is float32.
 
-    In steps of few tokens (`SIDE_BRANCH_MAX_TOKENS`), where a layer is a chain of short launches, the feed-forward
-    runs on a second stream beside the mixer: the two meet again before the layer returns, so a captured step holds
-    them as two branches of its graph. What the second stream allocates is read on the first only behind that meeting,
-    and written again only behind the next layer's parting, which follows the kernel that read it."""
+    In steps of few tokens (`base.SIDE_BRANCH_MAX_TOKENS`), where a layer is a chain of short launches, the feed-forward
+    runs on a second stream beside the mixer (`base.side_branch`): the two meet again before the layer returns, so a
+    captured step holds them as two branches of its graph. What the second stream allocates is read on the first only
+    behind that meeting, and written again only behind the next layer's parting, which follows the kernel that read it."""
 
     def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm | None = None, feed_forward: FeedForward | None = None,
                  residual_mult: float = 1.0, layer_scale: bool = False):
@@ -191,14 +178,11 @@ class ParallelBlock(Part):
         w2 = self.norm2.weight if self.feed_forward is not None else None
         stream, x1, x2 = ops.scaled_sum_norm(stream, terms, mult, self.norm1.weight, w2, self.norm1.eps, self.norm1.out_dtype)
         b = None
-        if self.feed_forward is not None and x1.is_cuda and 0 < x1.shape[0] <= SIDE_BRANCH_MAX_TOKENS:
-            import torch
-            main, side = torch.cuda.current_stream(x1.device), _side_stream(x1.device)
-            side.wait_stream(main)
-            with torch.cuda.stream(side), ops.second_workspace():
+        if self.feed_forward is not None and few_tokens(x1):
+            with side_branch(x1.device, 1) as branch:
                 b = self.feed_forward.forward(x2)
             out = [(self.mixer.forward(x1, step, cache, state), self.scale1)]
-            main.wait_stream(side)
+            branch.join()
         else:
             out = [(self.mixer.forward(x1, step, cache, state), self.scale1)]
             if self.feed_forward is not None:
