@@ -101,17 +101,11 @@ moe_logits_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict
   }
 }
 
-// The choice: a wave per token (4 tokens a workgroup). LDS per token: E scores, E working copies, the group scores.
-__global__ void __launch_bounds__(256)
-moe_select_kernel(const float* __restrict__ logits, int64_t T, int E, int top, int group_count, int group_keep,
-                  int32_t* __restrict__ ids, float* __restrict__ weights) {
-  extern __shared__ __align__(16) unsigned char route_lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
-  if (t >= T) return;
-  float* s = reinterpret_cast<float*>(route_lds) + (size_t)wave * (2 * E + group_count);
-  float* m = s + E;
-  float* gs = m + E;
+// The choice for one token by one wave. s, m: E floats of LDS each, gs: group_count floats.
+__device__ __forceinline__ void select_token(const float* __restrict__ logits, int64_t t, int E, int top, int group_count,
+                                             int group_keep, float* s, float* m, float* gs, int32_t* __restrict__ ids,
+                                             float* __restrict__ weights) {
+  const int lane = threadIdx.x & 63;
   const int per = E / group_count;
   float hi = -INFINITY;
   for (int e = lane; e < E; e += 64) { s[e] = logits[t * E + e]; hi = fmaxf(hi, s[e]); }
@@ -161,9 +155,22 @@ moe_select_kernel(const float* __restrict__ logits, int64_t T, int E, int top, i
   }
 }
 
+// The choice: a wave per token (4 tokens a workgroup). LDS per token: E scores, E working copies, the group scores.
+__global__ void __launch_bounds__(256)
+moe_select_kernel(const float* __restrict__ logits, int64_t T, int E, int top, int group_count, int group_keep,
+                  int32_t* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ __align__(16) unsigned char route_lds[];
+  const int wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float* s = reinterpret_cast<float*>(route_lds) + (size_t)wave * (2 * E + group_count);
+  select_token(logits, t, E, top, group_count, group_keep, s, s + E, s + 2 * E, ids, weights);
+}
+
 // logits: float32 [T, E] working memory.
 extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* w, int64_t T, int n, int E, int top,
-                            int group_count, int group_keep, float* logits, int32_t* ids, float* weights, hipStream_t stream) {
+                            int group_count, int group_keep, float* logits, int32_t* ids, float* weights, int select,
+                            hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && top >= 1 && top <= 64 && top <= E, "moe_route: %d experts, top %d", E, top);
   ME_CHECK(group_count >= 1 && E % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
@@ -175,14 +182,16 @@ extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* 
   ME_CHECK((size_t)TT * n * es <= 64 * 1024, "moe_route: a row of %d does not fit a workgroup's memory", n);
   const int64_t groups = (T + TT - 1) / TT;
   ME_CHECK(groups < (1ll << 31) && (T + 3) / 4 < (1ll << 31), "moe_route: too many tokens");
-  // few tokens: the experts spread over as many workgroups as possible; many: a workgroup keeps its rows for 32 experts
-  const int per_group = groups <= 64 ? 4 : 32;
+  // few tokens: the experts spread over as many workgroups as possible; many: a workgroup keeps its rows for 8 experts
+  // (two per wave: enough workgroups to a compute unit to hide each other's waits; 32 per workgroup took twice as long)
+  const int per_group = groups <= 64 ? 4 : 8;
   const dim3 grid((unsigned)groups, (unsigned)((E + per_group - 1) / per_group));
   if (dtype == ME_F32)
     moe_logits_kernel<float><<<grid, dim3(256), (size_t)TT * n * es, stream>>>((const float*)x, ldx, w, T, n, E, TT, per_group, logits);
   else
     moe_logits_kernel<bf16_t><<<grid, dim3(256), (size_t)TT * n * es, stream>>>((const bf16_t*)x, ldx, w, T, n, E, TT, per_group, logits);
   ME_LAUNCH_CHECK();
+  if (!select) return 0;           // the caller lets `me_moe_sort` choose (few tokens: one launch less)
   const size_t lds = (size_t)4 * (2 * E + group_count) * 4;
   ME_CHECK(lds <= 64 * 1024, "moe_route: %d experts do not fit a workgroup's memory", E);
   moe_select_kernel<<<dim3((unsigned)((T + 3) / 4)), dim3(256), lds, stream>>>(logits, T, E, top, group_count, group_keep, ids, weights);
@@ -193,11 +202,21 @@ extern "C" int me_moe_route(const void* x, int64_t ldx, int dtype, const float* 
 // ------------------------------------------------------------------ pairs by expert
 // One workgroup. order[p']: the pair at sorted place p'; offsets[e]: where expert e's pairs begin; tile_expert / tile_row:
 // expert and first sorted place of every tile of up to `tile_rows` pairs (expert -1: a tile nobody needs).
+// With `logits` (few tokens) the workgroup first makes the choice itself, a wave per token in turn, and writes ids and
+// weights: the launch of `moe_select` is saved.
 __global__ void __launch_bounds__(1024)
-moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, int tile_rows, int32_t* __restrict__ order,
-                int32_t* __restrict__ offsets, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row) {
+moe_sort_kernel(int32_t* __restrict__ ids, int P, int E, int max_tiles, int tile_rows, int32_t* __restrict__ order,
+                int32_t* __restrict__ offsets, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row,
+                const float* __restrict__ logits, float* __restrict__ weights, int top, int group_count, int group_keep) {
   __shared__ int count[MOE_MAX_EXPERTS], begin[MOE_MAX_EXPERTS + 1], tile_at[MOE_MAX_EXPERTS + 1], cursor[MOE_MAX_EXPERTS];
+  extern __shared__ __align__(16) unsigned char route_lds[];
   for (int e = threadIdx.x; e < E; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
+  if (logits) {
+    const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    float* s = reinterpret_cast<float*>(route_lds) + (size_t)wave * (2 * E + group_count);
+    for (int t = wave; t < P / top; t += waves) select_token(logits, t, E, top, group_count, group_keep, s, s + E, s + 2 * E, ids, weights);
+    __threadfence_block();
+  }
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
   __syncthreads();
@@ -224,13 +243,24 @@ moe_sort_kernel(const int32_t* __restrict__ ids, int P, int E, int max_tiles, in
   for (int i = tile_at[E] + threadIdx.x; i < max_tiles; i += blockDim.x) { tile_expert[i] = -1; tile_row[i] = 0; }
 }
 
-extern "C" int me_moe_sort(const int32_t* ids, int64_t P, int E, int max_tiles, int tile_rows, int32_t* order, int32_t* offsets,
-                           int32_t* tile_expert, int32_t* tile_row, hipStream_t stream) {
+// logits: null, or the router's float32 [T, E] with the choice still to be made (`me_moe_route` with select 0): ids and
+// weights are then written here (`moe_sort_chooses` says when that fits).
+extern "C" int me_moe_sort(int32_t* ids, int64_t P, int E, int max_tiles, int tile_rows, int32_t* order, int32_t* offsets,
+                           int32_t* tile_expert, int32_t* tile_row, const float* logits, float* weights, int top, int group_count,
+                           int group_keep, hipStream_t stream) {
   if (P == 0) return 0;
   ME_CHECK(E >= 1 && E <= MOE_MAX_EXPERTS && P < (1ll << 30), "moe_sort: %d experts, %lld pairs", E, (long long)P);
   ME_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_sort: tiles of 16, 64 or 128 rows");
   ME_CHECK(max_tiles >= P / tile_rows + (P < E ? P : E), "moe_sort: %d tiles cannot hold every expert's last tile", max_tiles);
-  moe_sort_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, (int)P, E, max_tiles, tile_rows, order, offsets, tile_expert, tile_row);
+  size_t lds = 0;
+  if (logits) {
+    ME_CHECK(weights && top >= 1 && top <= 64 && P % top == 0 && group_count >= 1 && E % group_count == 0 && group_keep >= 1 &&
+                 group_keep <= group_count && group_keep * (E / group_count) >= top, "moe_sort: bad routing sizes");
+    lds = (size_t)16 * (2 * E + group_count) * 4;
+    ME_CHECK(lds <= 40 * 1024, "moe_sort: %d experts are too many to choose here", E);
+  }
+  moe_sort_kernel<<<dim3(1), dim3(1024), lds, stream>>>(ids, (int)P, E, max_tiles, tile_rows, order, offsets, tile_expert, tile_row,
+                                                        logits, weights, top, group_count, group_keep);
   ME_LAUNCH_CHECK();
   return 0;
 }

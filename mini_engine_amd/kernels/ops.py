@@ -80,8 +80,8 @@ _CORE_PROTOS = {
     "me_scaled_sum_norm": [P, I, I, P, P, P, P, P, F, P, P, P, P, P, I, L, I, F, P],
     "me_softcap": [P, L, L, I, F, P],
     "me_qkv_prepare": [P, L, P, P, P, F, I, I, F, I, P, P, P, P, P, L, I, L, I, I, I, I, I, I, P, P, L, P],
-    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P, P],
-    "me_moe_sort": [P, L, I, I, I, P, P, P, P, P],
+    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P, I, P],
+    "me_moe_sort": [P, L, I, I, I, P, P, P, P, P, P, I, I, I, P],
     "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, P],
@@ -810,10 +810,31 @@ class HipBackend:
         weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
         logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
-                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), _stream())
+                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 1, _stream())
         return ids, weights
 
-    def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False, tile_rows: int | None = None) -> torch.Tensor:
+    def route_and_run_experts(self, x, router, top: int, group_count: int, group_keep: int, gate_up, down) -> torch.Tensor:
+        """`moe_route` and `routed_experts` behind it: float32 [top, T, hidden]. For the few tokens `moe_sort_chooses` admits,
+        the kernel that orders the pairs by expert makes the choice itself from the router's logits: one launch less in a
+        decode step's chain."""
+        T, n = x.shape
+        E = router.shape[0]
+        F = gate_up.shape[1] // 2
+        if not (moe_sort_chooses(T, E, group_count) and x.dtype == torch.bfloat16 and n % 8 == 0 and F % 8 == 0 and x.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0):
+            ids, weights = self.moe_route(x, router, top, group_count, group_keep)
+            return self.routed_experts(x, ids, weights, gate_up, down)
+        _check(x.stride(1) == 1 and router.dtype == torch.float32 and router.shape == (E, n) and router.is_contiguous(),
+               "moe_route: rows [T, n], router float32 [E, n]")
+        ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
+        weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+        logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
+        core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
+                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 0, _stream())
+        return self.routed_experts(x, ids, weights, gate_up, down, choose_from=(logits, group_count, group_keep))
+
+    def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False, tile_rows: int | None = None,
+                       choose_from=None) -> torch.Tensor:
         """Every token through its chosen gated experts: out[j, t] = weights[t, j] * W_down[e] (silu(W_gate[e] x_t) * (W_up[e] x_t)),
         e = ids[t, j]: float32 [top, T, hidden], one partial sum per choice for a consumer that adds them. x: [T, K];
         gate_up: [E, 2 F, K] (an expert's gate rows, then its up rows); down: [E, hidden, F]. bfloat16 with K and F in
@@ -843,8 +864,11 @@ class HipBackend:
         meta = torch.empty((Pn + E + 1 + 2 * max_tiles,), dtype=torch.int32, device=x.device)
         order, offsets = meta[:Pn], meta[Pn:Pn + E + 1]
         tile_expert, tile_row = meta[Pn + E + 1:Pn + E + 1 + max_tiles], meta[Pn + E + 1 + max_tiles:]
+        # choose_from (logits, group_count, group_keep): ids and weights are still empty and the sort kernel fills them
+        logits, gc, gk = choose_from if choose_from is not None else (None, 1, 1)
+        _check(choose_from is None or tiled, "routed_experts: the choice inside the sort kernel needs the tiled path")
         core().call("me_moe_sort", ids.data_ptr(), Pn, E, max_tiles, rows, order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
-                    tile_row.data_ptr(), _stream())
+                    tile_row.data_ptr(), _ptr(logits), weights.data_ptr(), top, int(gc), int(gk), _stream())
         core().call("me_moe_gate_up", x.data_ptr(), x.stride(0), gate_up.data_ptr(), order.data_ptr(), offsets.data_ptr(),
                     tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, rows, _stream())
         core().call("me_moe_down", act.data_ptr(), down.data_ptr(), order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
@@ -1315,6 +1339,16 @@ EXPERT_SKINNY_MAX_ROWS = 24       # mean rows per expert up to which the 16-row 
 EXPERT_LARGE_TILE_ROWS = 160      # ... from which tiles of 128 x 128 are taken
 
 
+SORT_CHOOSES_MAX_TOKENS = 64
+
+
+def moe_sort_chooses(T: int, E: int, group_count: int) -> bool:
+    """Whether the kernel that orders the (token, choice) pairs also makes the choice: up to SORT_CHOOSES_MAX_TOKENS tokens
+    (its one workgroup takes them 16 at a time, a wave each) and as many experts as leave its 16 waves their scratch
+    memory."""
+    return T <= SORT_CHOOSES_MAX_TOKENS and 16 * (2 * E + group_count) * 4 <= 40 * 1024
+
+
 def expert_tile_rows(T: int, top: int, E: int) -> int:
     """Rows per tile of the routed experts' kernels: 16 while an expert gets EXPERT_SKINNY_MAX_ROWS rows or fewer on
     average (decode steps and short portions: the step is the stream of the chosen experts' weights, and a tile of 16
@@ -1434,3 +1468,4 @@ def softcap_(*a, **k): return backend().softcap_(*a, **k)
 def qkv_prepare_store(*a, **k): return backend().qkv_prepare_store(*a, **k)
 def moe_route(*a, **k): return backend().moe_route(*a, **k)
 def routed_experts(*a, **k): return backend().routed_experts(*a, **k)
+def route_and_run_experts(*a, **k): return backend().route_and_run_experts(*a, **k)

@@ -39,8 +39,8 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x):
         E, F, h = self.num_experts, self.intermediate_size, self.hidden_size
-        ids, weights = ops.moe_route(x, self.router, self.top, self.group_count, self.group_keep)
-        routed = ops.routed_experts(x, ids, weights, self.gate_up.view(E, 2 * F, h), self.down.view(E, h, F))
+        routed = ops.route_and_run_experts(x, self.router, self.top, self.group_count, self.group_keep,
+                                           self.gate_up.view(E, 2 * F, h), self.down.view(E, h, F))
         if self.shared is None:
             return routed
         return routed, self.shared.forward(x)

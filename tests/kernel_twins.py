@@ -321,7 +321,12 @@ def moe_route(x, router, top, group_count=1, group_keep=1):
     return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20)).float()
 
 
-def routed_experts(x, ids, weights, gate_up, down, force_simple=False, tile_rows=None):
+def route_and_run_experts(x, router, top, group_count, group_keep, gate_up, down):
+    ids, weights = moe_route(x, router, top, group_count, group_keep)
+    return routed_experts(x, ids, weights, gate_up, down)
+
+
+def routed_experts(x, ids, weights, gate_up, down, force_simple=False, tile_rows=None, choose_from=None):
     T, K = x.shape
     top = ids.shape[1]
     F = gate_up.shape[1] // 2
@@ -414,3 +419,4 @@ class PlainBackend:
     qkv_prepare_store = staticmethod(qkv_prepare_store)
     moe_route = staticmethod(moe_route)
     routed_experts = staticmethod(routed_experts)
+    route_and_run_experts = staticmethod(route_and_run_experts)

@@ -132,3 +132,20 @@ def test_routed_experts(dtype, simple, E, top, F, K, T):
     close(got, want, 2e-5 if dtype == torch.float32 else 1.5e-2)
     if dtype == torch.bfloat16:
         close(got.sum(0), want.sum(0), 1e-2)
+
+
+@pytest.mark.parametrize("E,top,count,keep,F,K", [(12, 3, 3, 2, 48, 160), (32, 4, 4, 2, 384, 1024), (256, 8, 8, 4, 64, 512), (512, 2, 1, 1, 16, 64)])
+def test_route_and_run_experts(E, top, count, keep, F, K):
+    """Few tokens: the kernel that orders the pairs makes the choice itself (up to the expert count that fits it); the
+    result is that of the two operations one after the other."""
+    torch.manual_seed(E + K)
+    router = torch.randn(E, K, device=DEV) * (3.0 / K ** 0.5)
+    gate_up = (torch.randn(E, 2 * F, K, device=DEV) * K ** -0.5).bfloat16()
+    down = (torch.randn(E, K, F, device=DEV) * F ** -0.5).bfloat16()
+    for T in (1, 7, 64, 65):
+        x = torch.randn(T, K, device=DEV).bfloat16()
+        got = hip().route_and_run_experts(x, router, top, count, keep, gate_up, down)
+        ids, w = hip().moe_route(x, router, top, count, keep)
+        want = hip().routed_experts(x, ids, w, gate_up, down)
+        assert torch.equal(got, want), f"T={T}: the fused choice differs from the separate one"
+    assert ops.moe_sort_chooses(64, 256, 8) and not ops.moe_sort_chooses(65, 32, 1) and not ops.moe_sort_chooses(8, 512, 1)
