@@ -60,9 +60,19 @@ moe_logits_kernel(const TX* __restrict__ x, int64_t ldx, const float* __restrict
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t t0 = (int64_t)blockIdx.x * TT;
   const int live = (int)min((int64_t)TT, T - t0);
-  for (int i = threadIdx.x; i < TT * n; i += blockDim.x) {
-    const int tt = i / n, k = i - tt * n;
-    xs[i] = tt < live ? x[(t0 + tt) * ldx + k] : from_f32<TX>(0.f);
+  constexpr int EPV = 16 / sizeof(TX);       // elements of a 16-byte piece
+  if (n % EPV == 0 && ldx % EPV == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    const int pieces = n / EPV;
+    for (int i = threadIdx.x; i < TT * pieces; i += blockDim.x) {
+      const int tt = i / pieces, c = i - tt * pieces;
+      const uint4 v = tt < live ? *reinterpret_cast<const uint4*>(x + (t0 + tt) * ldx + c * EPV) : make_uint4(0u, 0u, 0u, 0u);
+      *reinterpret_cast<uint4*>(xs + tt * n + c * EPV) = v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < TT * n; i += blockDim.x) {
+      const int tt = i / n, k = i - tt * n;
+      xs[i] = tt < live ? x[(t0 + tt) * ldx + k] : from_f32<TX>(0.f);
+    }
   }
   __syncthreads();
   const int e0 = blockIdx.y * experts_per_group, e1 = min(E, e0 + experts_per_group);
