@@ -230,3 +230,27 @@ def test_command_line_on_a_folder_of_this_design(negosun_folders, plain_backend,
         for tok in g:
             assert tok == int(N.plain_logits(folder, seq)[-1].argmax())
             seq.append(tok)
+
+
+def test_launch_rules_of_the_routed_experts():
+    """Whatever the step: tiles of a size the kernels are built for, small ones while experts get few rows, and the tile
+    count the launches are sized by holds every expert's tiles however the pairs fall; the kernel that orders the pairs
+    chooses only for steps and expert counts that fit its one workgroup."""
+    from mini_engine_amd.kernels import ops
+    import random
+    rng = random.Random(1)
+    for _ in range(3000):
+        T, top, E = rng.choice((1, 2, 7, 64, 65, 300, 2048, 16384)), rng.choice((1, 2, 4, 8)), rng.choice((2, 8, 32, 60, 256))
+        top = min(top, E)
+        rows = ops.expert_tile_rows(T, top, E)
+        assert rows in (16, 64, 128)
+        assert rows == 16 or T * top > 16 * E and (rows == 64 or T * top >= 128 * E)
+        # the worst split of the pairs over the experts: every expert that has pairs ends in a tile that is not full
+        counts = [0] * E
+        for _ in range(T * top if T * top < 200 else 200):
+            counts[rng.randrange(E)] += max(1, T * top // 200)
+        counts[0] += T * top - sum(counts) if sum(counts) <= T * top else 0
+        if sum(counts) == T * top:
+            assert sum(-(-c // rows) for c in counts) <= T * top // rows + min(E, T * top)
+    assert ops.moe_sort_chooses(1, 32, 4) and ops.moe_sort_chooses(64, 256, 8)
+    assert not ops.moe_sort_chooses(65, 32, 4) and not ops.moe_sort_chooses(4, 1024, 1)

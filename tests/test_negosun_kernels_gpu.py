@@ -78,7 +78,7 @@ def test_qkv_prologue(dtype, Hq, Hkv, D, n, nv, page):
     slots = torch.randperm(pages * page, device=DEV)[:T].to(torch.int32)
     slots[3] = -1
     lam = torch.tensor(0.3, device=DEV)
-    for mix, temperature, normed in ((0, None, True), (1, (0.5, 7), True), (2, (0.25, 128), True), (2, None, False)):
+    for mix, temperature, normed in ((0, None, True), (1, (0.5, 7), True), (2, (0.25, 96), True), (2, None, False)):
         got, want = [], []
         for be, keep in ((hip(), got), (twin, want)):
             kc = torch.zeros(pages, Hkv, page, D, device=DEV, dtype=dtype)
