@@ -372,12 +372,19 @@ moe_tile_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
 #pragma unroll
       for (int i = 0; i < MI / 2; ++i) {
         const int f = n0 + wn * (TN / 4) + 16 * i + 4 * g;
+        bf16x4 r;
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (f + q < N) {
-            const float gate = acc[i][j][q];
-            o[f + q] = from_f32<bf16_t>(gate / (1.f + __expf(-gate)) * acc[i + MI / 2][j][q]);
-          }
+        for (int q = 0; q < 4; ++q) {
+          const float gate = acc[i][j][q];
+          r[q] = from_f32<bf16_t>(gate / (1.f + __expf(-gate)) * acc[i + MI / 2][j][q]);
+        }
+        if (f + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<bf16x4*>(o + f) = r;          // 4 neighbours, 8 bytes
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (f + q < N) o[f + q] = r[q];
+        }
       }
     } else {
       const int pair = order[p];
@@ -387,9 +394,13 @@ moe_tile_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
         const int f = n0 + wn * (TN / 2) + 16 * i + 4 * g;
+        if (f + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<float4*>(o + f) = make_float4(acc[i][j][0] * pw, acc[i][j][1] * pw, acc[i][j][2] * pw, acc[i][j][3] * pw);
+        } else {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (f + q < N) o[f + q] = acc[i][j][q] * pw;
+          for (int q = 0; q < 4; ++q)
+            if (f + q < N) o[f + q] = acc[i][j][q] * pw;
+        }
       }
     }
   }

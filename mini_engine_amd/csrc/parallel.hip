@@ -235,6 +235,8 @@ qkv_prepare_kernel(const float* __restrict__ rows, int64_t row_stride, const flo
     }
   }
   const float lam = mix == 2 ? lambda[0] : 0.f;
+  // (Writing a group of 8 tokens' values as 16-byte pieces by the workgroup of the group's first token was measured: that
+  // workgroup then does eight tokens' work while seven idle, 54 -> 89 us for 2,048 tokens of 8 heads of 128.)
   for (int i = threadIdx.x; i < wk; i += blockDim.x) {
     const int h = i / D, d = i - h * D;
     float v = r[wq + wk + i] + (bias ? bias[wq + wk + i] : 0.f);

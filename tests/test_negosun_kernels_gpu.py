@@ -75,10 +75,15 @@ def test_qkv_prologue(dtype, Hq, Hkv, D, n, nv, page):
     bias = torch.randn(width, device=DEV) * mask
     qw, kw = torch.rand(Hq * D, device=DEV) + 0.5, torch.rand(Hkv * D, device=DEV) + 0.5
     positions = torch.randint(0, 1000, (T,), device=DEV, dtype=torch.int32)
-    slots = torch.randperm(pages * page, device=DEV)[:T].to(torch.int32)
-    slots[3] = -1
+    scattered = torch.randperm(pages * page, device=DEV)[:T].to(torch.int32)
+    scattered[3] = -1
+    # a prompt's portions: 24 consecutive places from the start of a page (three groups of 8 tokens, which the kernel writes
+    # with vector stores, over a page's border), then runs that start inside a page or at a token that starts no group
+    runs = torch.cat([torch.arange(a, a + n) for a, n in ((5 * page, 24), (3, 9), (12 * page, 10))])
+    portions = torch.cat((runs, torch.full((T - runs.numel(),), -1))).to(torch.int32).to(DEV)
     lam = torch.tensor(0.3, device=DEV)
-    for mix, temperature, normed in ((0, None, True), (1, (0.5, 7), True), (2, (0.25, 96), True), (2, None, False)):
+    cases = ((0, None, True), (1, (0.5, 7), True), (2, (0.25, 96), True), (2, None, False))
+    for slots, (mix, temperature, normed) in ((s, c) for s in (scattered, portions) for c in cases):
         got, want = [], []
         for be, keep in ((hip(), got), (twin, want)):
             kc = torch.zeros(pages, Hkv, page, D, device=DEV, dtype=dtype)
