@@ -71,14 +71,22 @@ CONFIGS = {
         _layer(3, 1, 32, 16, 0.2, temp=(0.5, 64), v_mix=True, moe=_moe(4, 2, 40, shared=16)),
     ]),
 }
+# mid sizes: heads of 64 on the matrix-core attention kernels without padding, 64 experts in eight groups of which three are
+# kept, six per token, rows in whole 16-byte pieces (the tiled expert kernels in bfloat16); layers that differ
+CONFIGS["mid"] = _model(1000, 256, 1e-6, 0.7, 12.0, [
+    _layer(8, 4, 64, 64, 0.125, temp=(0.4, 32), v_mix=True, moe=_moe(64, 6, 32, groups=(8, 3), shared=64)),
+    _layer(4, 2, 64, 128, 0.125, v_mix=True),
+    _layer(8, 4, 64, 64, 0.125, temp=(0.4, 32), v_mix=True, moe=_moe(24, 2, 48, groups=(4, 1))),
+    _layer(8, 8, 32, 32, 0.2, v_mix=True, moe=_moe(10, 3, 40, shared=16)),
+])
 # the layer sizes of a real model (heads of 128, experts of 256 in four groups), two layers: the kernel forms that the
 # small widths above never reach
 CONFIGS["real"] = _model(1000, 512, 1e-6, 0.6, 25.0, [
     _layer(8, 2, 128, 128, 128 ** -0.5, temp=(0.1, 256), v_mix=True, moe=_moe(16, 4, 256, groups=(4, 2), shared=512)),
     _layer(8, 2, 128, 128, 128 ** -0.5, temp=(0.1, 256), v_mix=True, moe=_moe(16, 4, 256, groups=(4, 2), shared=512)),
 ])
-SEEDS = {"trio": 21, "solo": 22, "late": 23, "far": 24, "real": 25}
-PAGE = {"trio": 8, "solo": 16, "late": 16, "far": 16, "real": 16}
+SEEDS = {"trio": 21, "solo": 22, "late": 23, "far": 24, "real": 25, "mid": 26}
+PAGE = {"trio": 8, "solo": 16, "late": 16, "far": 16, "real": 16, "mid": 16}
 SHARPEN, BIAS_UP, ROUTER_UP = 3.0, 15.0, 40.0
 
 

@@ -60,6 +60,12 @@ def test_far_keys_and_temperature_steps(env):
     N.far_keys(env)
 
 
+@pytest.mark.parametrize("case", [N.whole, N.portions, N.batch_against_alone], ids=lambda c: c.__name__)
+def test_mid_sizes(env, case):
+    """Heads of 64 without padding, 64 experts of which six are used, the tiled expert kernels in bfloat16."""
+    case(env, "mid")
+
+
 def test_real_layer_sizes(negosun_folders):
     N.real_sizes(Env(negosun_folders, torch.float32), Env(negosun_folders, torch.bfloat16))
 
